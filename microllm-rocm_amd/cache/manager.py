@@ -19,7 +19,7 @@ from typing import Dict, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
-from .needs import Binding, CacheNeed, PagedBinding, PagedKVNeed, StateBinding, StateNeed
+from .needs import Binding, CacheNeed, CompositeBinding, CompositeNeed, PagedBinding, PagedKVNeed, StateBinding, StateNeed
 from .pages import OutOfPages, PagePool, SlotPool
 
 RELEASED = -1  # block-table entry of a page that a window has passed
@@ -95,12 +95,17 @@ class CacheManager:
         self.requests: Dict[Hashable, RequestCache] = {}
         self._bindings: List[Optional[Binding]] = [None] * len(needs)
         self._slot_storage: List[tuple] = []        # (need, storage) of every run entry that keeps state in slots
+        self._slot_needs: List[CacheNeed] = []      # the same needs, also where the manager only keeps books
         by_need: Dict[CacheNeed, CacheGroup] = {}
-        for entry, need in enumerate(needs):
-            if reads[entry] is not None or need is None:
-                continue
+
+        def provide(entry: int, need: Optional[CacheNeed]) -> Optional[Binding]:
+            """Storage and binding for one need of run entry ``entry``; a composite need gets each part's."""
+            if need is None:
+                return None
             if not isinstance(need, CacheNeed):
                 raise TypeError(f"run entry {entry} declares an unknown cache need {need!r}")
+            if isinstance(need, CompositeNeed):
+                return CompositeBinding(need, True, tuple(provide(entry, part) for part in need.parts))
             if need.paged:
                 if device is not None:
                     need.check_page_size(page_size)   # the layout on the device may ask more of a page than the books do
@@ -112,12 +117,16 @@ class CacheManager:
                     by_need[need] = group
                 group.entries.append(entry)
                 storage = need.allocate_pages(group.pool.num_pages, page_size, dtype, device) if device is not None else None
-                self._bindings[entry] = need.bind(group.index, storage, True)
-            else:
-                storage = need.allocate_slots(max_requests, dtype, device) if device is not None else None
-                if storage is not None:
-                    self._slot_storage.append((need, storage))
-                self._bindings[entry] = need.bind(None, storage, True)
+                return need.bind(group.index, storage, True)
+            storage = need.allocate_slots(max_requests, dtype, device) if device is not None else None
+            if storage is not None:
+                self._slot_storage.append((need, storage))
+            self._slot_needs.append(need)
+            return need.bind(None, storage, True)
+
+        for entry, need in enumerate(needs):
+            if reads[entry] is None and need is not None:
+                self._bindings[entry] = provide(entry, need)
         for entry, source in enumerate(reads):
             if source is None:
                 continue
@@ -131,7 +140,7 @@ class CacheManager:
     def has_state(self) -> bool:
         """Whether any run entry keeps per-request state of fixed size (which, unlike pages, a failed step cannot
         simply leave behind)."""
-        return any(binding is not None and not binding.need.paged and binding.owned for binding in self._bindings)
+        return bool(self._slot_needs)
 
     def bindings(self) -> List[object]:
         return list(self._bindings)
@@ -234,6 +243,20 @@ class CacheManager:
         self.slots.give([request.slot])
         request.closed = True
 
+    # ---- state slots around a run that must not count -----------------------------------------
+    def save_slots(self, slots: Sequence[int]) -> list:
+        """Copies of what the given request slots hold in every run entry's state (for ``restore_slots``)."""
+        if not self._slot_storage or not len(slots):
+            return []
+        index = torch.as_tensor(sorted(set(int(slot) for slot in slots)), dtype=torch.int64, device=self.device)
+        return [(storage, index, storage.index_select(0, index)) for _, storage in self._slot_storage
+                if isinstance(storage, torch.Tensor)]
+
+    @staticmethod
+    def restore_slots(saved: list) -> None:
+        for storage, index, values in saved:
+            storage.index_copy_(0, index, values)
+
     # ---- accounting ----------------------------------------------------------------------
     def free_pages(self) -> List[int]:
         return [group.pool.num_free for group in self.groups]
@@ -246,8 +269,7 @@ class CacheManager:
 
     def state_bytes(self) -> int:
         """Bytes of the slots of every run entry that keeps per-request state, for all request slots."""
-        return sum(self.max_requests * binding.need.bytes_per_request(self.dtype) for binding in self._bindings
-                   if binding is not None and not binding.need.paged and binding.owned)
+        return sum(self.max_requests * need.bytes_per_request(self.dtype) for need in self._slot_needs)
 
     def allocated_bytes(self) -> int:
         return sum(self.bytes_per_page(group) * group.pool.num_pages for group in self.groups)

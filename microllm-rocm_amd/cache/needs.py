@@ -7,8 +7,10 @@ storage, and hands the mixer whatever ``bind`` returns. Needs that compare equal
 pages and one block table per request. A new kind of cache payload (one latent vector a token, keys alone, keys
 and values of different widths) is a new subclass, defined wherever its mixer is; nothing here lists kinds.
 
-The two kinds this package's own parts use are here: ``PagedKVNeed`` (keys and values in the tile order the MFMA
-attention kernels read, see ``cache.layout``) and ``StateNeed`` (a tensor per request, zero when it opens).
+The kinds this package's own parts use are here: ``PagedKVNeed`` (keys and values in the tile order the MFMA
+attention kernels read, see ``cache.layout``), ``PagedKeyValueNeed`` (keys and values of widths of their own in plain
+pages), ``StateNeed`` (a tensor per request, zero when it opens) and ``CompositeNeed`` (several of these for one
+mixer: one that runs an attention beside a layer with state asks for both).
 The reference has one ``[slots, kv_heads, capacity, head_dim]`` tensor per layer and nothing else
 (src/inference/kv_cache.cpp:11-64).
 """
@@ -119,6 +121,34 @@ class PagedBinding(Binding):
         return [tensor for tensor in (self.k, self.v) if tensor is not None]
 
 
+# ---- keys and values of different widths, in plain pages ---------------------------------------------------
+@dataclass(frozen=True)
+class PagedKeyValueNeed(CacheNeed):
+    """Keys ``[page, position, kv_head, key_dim]`` and values ``[page, position, kv_head, value_dim]``: the two widths
+    are free, and a position's row is contiguous (what the attention with a bias by distance reads)."""
+    kv_heads: int
+    key_dim: int
+    value_dim: int
+    window: Optional[int] = None
+    paged = True
+
+    def check_page_size(self, page_size: int) -> None:
+        if page_size <= 0:
+            raise ValueError("page_size must be positive")
+
+    def allocate_pages(self, num_pages, page_size, dtype, device):
+        k = torch.zeros((num_pages, page_size, self.kv_heads, self.key_dim), dtype=dtype, device=device)
+        v = torch.zeros((num_pages, page_size, self.kv_heads, self.value_dim), dtype=dtype, device=device)
+        return k, v
+
+    def bytes_per_position(self, dtype):
+        return self.kv_heads * (self.key_dim + self.value_dim) * _element_size(dtype)
+
+    def bind(self, group, storage, owned):
+        k, v = storage if storage is not None else (None, None)
+        return PagedBinding(self, owned, group, k, v)
+
+
 # ---- per-request state of fixed size -------------------------------------------------------------
 @dataclass(frozen=True)
 class StateNeed(CacheNeed):
@@ -149,3 +179,50 @@ class StateBinding(Binding):
 
     def tensors(self):
         return [self.state] if self.state is not None else []
+
+
+# ---- several needs of one mixer ----------------------------------------------------------------------------
+@dataclass(frozen=True)
+class CompositeNeed(CacheNeed):
+    """What a mixer made of several mixers keeps: each part's need, in the parts' order (None for a part that keeps
+    nothing). The manager gives every part what it would give a run entry with that need alone (paged parts join
+    the groups of equal needs, state parts get slots) and hands the mixer a ``CompositeBinding``."""
+    parts: Tuple[Optional[CacheNeed], ...]
+
+    def flat(self) -> List[CacheNeed]:
+        """Every need that is no composite itself, in order."""
+        found: List[CacheNeed] = []
+        for part in self.parts:
+            if isinstance(part, CompositeNeed):
+                found += part.flat()
+            elif part is not None:
+                found.append(part)
+        return found
+
+
+@dataclass
+class CompositeBinding(Binding):
+    """``parts[i]`` is the binding of the i-th part's need (None where that part keeps nothing)."""
+    parts: Tuple[Optional[Binding], ...] = ()
+
+    def tensors(self):
+        return [tensor for part in self.parts if part is not None for tensor in part.tensors()]
+
+    def shared(self):
+        return dataclasses.replace(self, owned=False, parts=tuple(part.shared() if part is not None else None for part in self.parts))
+
+
+def flat_needs(need: Optional[CacheNeed]) -> List[CacheNeed]:
+    """The needs behind ``need`` that are no composites: what memory estimates and byte counts add up."""
+    if need is None:
+        return []
+    return need.flat() if isinstance(need, CompositeNeed) else [need]
+
+
+def flat_bindings(binding: Optional[Binding]) -> List[Binding]:
+    """The bindings behind ``binding`` that are no composites."""
+    if binding is None:
+        return []
+    if isinstance(binding, CompositeBinding):
+        return [inner for part in binding.parts for inner in flat_bindings(part)]
+    return [binding]

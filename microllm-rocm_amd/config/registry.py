@@ -21,6 +21,9 @@ class Architecture:
     config_from_dict: Callable[[Mapping[str, Any]], Any]
     build_spec: Callable[[Any], Any]                      # configuration -> ModelSpec
     init_rules: Optional[Callable[[Any], Any]] = None     # configuration -> rules for random weights
+    # (configuration, {tensor name: shape} of the model's files) -> the configuration with the sizes that no key
+    # of config.json gives and only a tensor's shape does; None where config.json says everything
+    complete_config: Optional[Callable[[Any, Mapping[str, Any]], Any]] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
@@ -54,6 +57,8 @@ def architecture_named(name: str) -> Architecture:
 
 
 def architecture_of(source: Mapping[str, Any]) -> Architecture:
+    if "architectures" not in source and isinstance(source.get("architecture"), str):
+        return architecture_named(source["architecture"])     # some designs name themselves with one string
     names = fields.string_list(source, "architectures")
     if len(names) != 1:
         raise ConfigError(f"config key architectures must name exactly one architecture, got {names!r}")
@@ -67,4 +72,8 @@ def load_config(folder_or_file: str):
         path = os.path.join(path, "config.json")
     source = fields.read_json_object(path)
     architecture = architecture_of(source)
-    return architecture, architecture.config_from_dict(source)
+    config = architecture.config_from_dict(source)
+    if architecture.complete_config is not None and os.path.isdir(folder_or_file):
+        from ..weights.safetensors_io import tensor_shapes
+        config = architecture.complete_config(config, tensor_shapes(folder_or_file))
+    return architecture, config

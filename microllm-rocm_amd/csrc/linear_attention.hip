@@ -1,0 +1,184 @@
+// Gated linear attention: a matrix of state per head and request, decayed per key channel and carried from token
+// to token.
+//
+//   S_t = diag(a_t) S_(t-1) + k_t v_t^T        (S: [key_dim, value_dim], a_t in (0, 1) per key channel)
+//   o_t = S_t^T q_t
+//
+// with a_t = sigmoid(z_t)^(1 / tau), z_t = A2 (low-rank input) + b. Three kernels: the decays of a step's tokens
+// (all tokens at once), the walk over each request's tokens in order (the state's columns are independent, so a
+// request's head is spread over workgroups by value channel), and the norm and gate of the results. State, decays
+// and everything the walk touches are float32, whatever the engine's element type.
+#include "common.h"
+#include "microllm_hip.h"
+
+namespace mll {
+
+constexpr int kStateRowsALane = 8;     // key channels a lane keeps of its column of the state
+
+// decay[t, c] = exp(log_sigmoid(z) / tau), z = bias[c] + sum_r a2[c, r] * low[t, r]
+template <typename W>
+__global__ void gla_decay_kernel(const float* __restrict__ proj, int64_t proj_stride, int low_offset, int rank,
+                                 const W* __restrict__ a2, const float* __restrict__ bias, float inv_tau,
+                                 float* __restrict__ decay, int channels) {
+    const int token = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    const float* low = proj + static_cast<int64_t>(token) * proj_stride + low_offset;
+    float z = bias ? bias[c] : 0.0f;
+    for (int r = 0; r < rank; ++r) z = fmaf(to_float(a2[static_cast<int64_t>(c) * rank + r]), low[r], z);
+    // log(sigmoid(z)) = -(max(-z, 0) + log1p(exp(-|z|)))
+    const float log_sigmoid = -(fmaxf(-z, 0.0f) + log1pf(expf(-fabsf(z))));
+    decay[static_cast<int64_t>(token) * channels + c] = expf(log_sigmoid * inv_tau);
+}
+
+// One wave a (request, head, group of value channels). lane = column_in_group * lanes_a_column + r; lane r of a
+// column keeps key channels r, r + lanes_a_column, ... (kStateRowsALane of them).
+__global__ void __launch_bounds__(kWave)
+gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
+                const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
+                const int32_t* __restrict__ slots, float* __restrict__ out, int heads, int key_dim, int value_dim,
+                int lanes_a_column, float q_scale) {
+    const int seq = blockIdx.x;
+    const int head = blockIdx.y;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    if (last <= first) return;       // a request that pads the step brings no tokens
+    const int lane = threadIdx.x;
+    const int r = lane % lanes_a_column;
+    const int column = blockIdx.z * (kWave / lanes_a_column) + lane / lanes_a_column;
+    const bool live = column < value_dim;
+    const int safe_column = live ? column : 0;
+    const int slot = slots[seq];
+    float* mine = state + ((static_cast<int64_t>(slot) * heads + head) * key_dim) * value_dim + safe_column;
+    float s[kStateRowsALane];
+#pragma unroll
+    for (int m = 0; m < kStateRowsALane; ++m) {
+        const int i = r + m * lanes_a_column;
+        s[m] = i < key_dim ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
+    }
+    const int channels = heads * key_dim;
+    float a_next[kStateRowsALane], k_next[kStateRowsALane], q_next[kStateRowsALane], v_next;
+    auto fetch = [&](int token) {
+        const float* row = proj + static_cast<int64_t>(token) * proj_stride;
+        const float* decays = decay + static_cast<int64_t>(token) * channels + head * key_dim;
+#pragma unroll
+        for (int m = 0; m < kStateRowsALane; ++m) {
+            const int i = r + m * lanes_a_column;
+            const bool in = i < key_dim;
+            a_next[m] = in ? decays[i] : 0.0f;
+            k_next[m] = in ? row[k_offset + head * key_dim + i] : 0.0f;
+            q_next[m] = in ? row[q_offset + head * key_dim + i] : 0.0f;
+        }
+        v_next = row[v_offset + head * value_dim + safe_column];
+    };
+    fetch(first);
+    for (int token = first; token < last; ++token) {
+        float a[kStateRowsALane], k[kStateRowsALane], q[kStateRowsALane];
+#pragma unroll
+        for (int m = 0; m < kStateRowsALane; ++m) a[m] = a_next[m], k[m] = k_next[m], q[m] = q_next[m];
+        const float v = v_next;
+        if (token + 1 < last) fetch(token + 1);
+        float partial = 0.0f;
+#pragma unroll
+        for (int m = 0; m < kStateRowsALane; ++m) {
+            s[m] = fmaf(a[m], s[m], k[m] * v);
+            partial = fmaf(s[m], q[m] * q_scale, partial);
+        }
+        for (int offset = 1; offset < lanes_a_column; offset <<= 1) partial += __shfl_xor(partial, offset, kWave);
+        if (live && r == 0) out[(static_cast<int64_t>(token) * heads + head) * value_dim + column] = partial;
+    }
+    if (!live) return;
+#pragma unroll
+    for (int m = 0; m < kStateRowsALane; ++m) {
+        const int i = r + m * lanes_a_column;
+        if (i < key_dim) mine[static_cast<int64_t>(i) * value_dim] = s[m];
+    }
+}
+
+// out[t, head, :] = rms_norm(o[t, head, :]) * weight * silu(gate[t, head, :]) * out_scale; one wave a (token, head).
+template <typename T>
+__global__ void __launch_bounds__(kWave)
+gla_gate_kernel(const float* __restrict__ o, const float* __restrict__ proj, int64_t proj_stride, int gate_offset,
+                const float* __restrict__ weight, float eps, T* __restrict__ out, int64_t out_stride, int heads,
+                int value_dim, float out_scale) {
+    const int token = blockIdx.x / heads;
+    const int head = blockIdx.x % heads;
+    const int lane = threadIdx.x;
+    const float* row = o + (static_cast<int64_t>(token) * heads + head) * value_dim;
+    const float* gate = proj + static_cast<int64_t>(token) * proj_stride + gate_offset + head * value_dim;
+    float squares = 0.0f;
+    for (int c = lane; c < value_dim; c += kWave) squares += row[c] * row[c];
+    const float factor = 1.0f / sqrtf(wave_sum(squares) / static_cast<float>(value_dim) + eps);
+    T* to = out + static_cast<int64_t>(token) * out_stride + head * value_dim;
+    for (int c = lane; c < value_dim; c += kWave) {
+        const float g = gate[c];
+        const float silu = g / (1.0f + expf(-g));
+        to[c] = from_float<T>(row[c] * factor * weight[c] * silu * out_scale);
+    }
+}
+
+}  // namespace mll
+
+using namespace mll;
+
+extern "C" {
+
+int mll_gla_decay(const float* proj, int64_t proj_stride, int low_offset, int rank, const void* a2, int a2_dtype,
+                  const float* bias, float tau, float* decay, int n_tokens, int channels, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && channels > 0 && rank > 0 && tau > 0.0f, "gla_decay: sizes and tau must be positive");
+    MLL_REQUIRE(low_offset >= 0 && low_offset + rank <= proj_stride, "gla_decay: the low-rank input lies outside its row");
+    if (n_tokens == 0) return 0;
+    MLL_REQUIRE(n_tokens <= 65535, "gla_decay: more than 65535 tokens in one call");
+    const dim3 grid((channels + 127) / 128, n_tokens);
+    if (a2_dtype == kF32) {
+        gla_decay_kernel<float><<<grid, 128, 0, stream>>>(proj, proj_stride, low_offset, rank, static_cast<const float*>(a2), bias,
+                                                         1.0f / tau, decay, channels);
+    } else if (a2_dtype == kBF16) {
+        gla_decay_kernel<bf16><<<grid, 128, 0, stream>>>(proj, proj_stride, low_offset, rank, static_cast<const bf16*>(a2), bias,
+                                                        1.0f / tau, decay, channels);
+    } else {
+        return fail("gla_decay: unknown weight dtype");
+    }
+    return check_launch("gla_decay");
+}
+
+int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset, const float* decay,
+                 float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
+                 int value_dim, float q_scale, hipStream_t stream) {
+    MLL_REQUIRE(n_seqs >= 0 && heads > 0 && key_dim > 0 && value_dim > 0, "gla_scan: sizes must be positive");
+    MLL_REQUIRE(key_dim <= kStateRowsALane * kWave, "gla_scan: key heads wider than 512 are not supported");
+    MLL_REQUIRE(q_offset >= 0 && k_offset >= 0 && v_offset >= 0 && q_offset + heads * key_dim <= proj_stride &&
+                    k_offset + heads * key_dim <= proj_stride && v_offset + heads * value_dim <= proj_stride,
+                "gla_scan: a projection lies outside its row");
+    if (n_seqs == 0) return 0;
+    int lanes_a_column = 1;
+    while (lanes_a_column * kStateRowsALane < key_dim) lanes_a_column <<= 1;
+    const int columns_a_wave = kWave / lanes_a_column;
+    MLL_REQUIRE(n_seqs <= 65535 * 32 && heads <= 65535, "gla_scan: too many requests or heads for one launch");
+    const dim3 grid(n_seqs, heads, (value_dim + columns_a_wave - 1) / columns_a_wave);
+    gla_scan_kernel<<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens, slots,
+                                               out, heads, key_dim, value_dim, lanes_a_column, q_scale);
+    return check_launch("gla_scan");
+}
+
+int mll_gla_gate(const float* o, const float* proj, int64_t proj_stride, int gate_offset, const float* weight, float eps,
+                 void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int value_dim, float out_scale,
+                 hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && heads > 0 && value_dim > 0 && eps > 0.0f, "gla_gate: sizes and eps must be positive");
+    MLL_REQUIRE(gate_offset >= 0 && gate_offset + heads * value_dim <= proj_stride, "gla_gate: the gate lies outside its row");
+    MLL_REQUIRE(out_stride >= static_cast<int64_t>(heads) * value_dim, "gla_gate: the output rows overlap");
+    if (n_tokens == 0) return 0;
+    const int64_t blocks = static_cast<int64_t>(n_tokens) * heads;
+    MLL_REQUIRE(blocks < (1ll << 31), "gla_gate: too many rows for one launch");
+    if (dtype == kF32) {
+        gla_gate_kernel<float><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(o, proj, proj_stride, gate_offset, weight, eps,
+                                                                                   static_cast<float*>(out), out_stride, heads, value_dim, out_scale);
+    } else if (dtype == kBF16) {
+        gla_gate_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(o, proj, proj_stride, gate_offset, weight, eps,
+                                                                                  static_cast<bf16*>(out), out_stride, heads, value_dim, out_scale);
+    } else {
+        return fail("gla_gate: unknown dtype");
+    }
+    return check_launch("gla_gate");
+}
+
+}  // extern "C"

@@ -214,4 +214,72 @@ int mll_sample(const float* logits, const float* temperature, const int32_t* top
                hipStream_t stream);
 int64_t mll_sample_workspace(int n_rows, int vocab);
 
+// ---- several copies of the residual stream, a norm with a mean, a sinusoidal position vector ----------------
+
+// out[t, :] = table[ids[t], :] + wave(positions[t]) in float32, where entry 2i of the wave is
+// sin(p * base^(-2i / width)) and entry 2i + 1 the cosine of the same angle (the angle in float64).
+int mll_embedding_sinusoid(const void* table, int table_dtype, const int32_t* ids, const int32_t* positions, float* out,
+                           int n_tokens, int width, int vocab, double base, hipStream_t stream);
+
+// out[t, c, :] = in[t, :] for every copy c: float32 [n_tokens][copies][width].
+int mll_stream_copies(const float* in, float* out, int n_tokens, int width, int copies, hipStream_t stream);
+
+// x is float32 [rows][streams][width]. For i < n_rows, r = rows ? rows[i] : i:
+//   if y:  d = sum of y's n_parts parts at row r (float32 [width], parts part_stride elements apart);
+//          x'_t = sum_s mix[s * streams + t] * x_s + give[t] * d  for every t (mix null: x'_t = x_t + give[t] * d;
+//          give null: ones); with write_x the new rows replace the old ones;
+//   u = sum_t take[t] * x'_t  (take null: ones);
+//   out[i] = (u - mean(u)) / sqrt(var(u) + eps) * weight, or with rms: u / sqrt(mean(u^2) + eps) * weight.
+// out null: only the streams are written. out has element type `dtype`; mix, give, take and weight are float32.
+int mll_stream_norm(float* x, const float* y, int n_parts, int64_t part_stride, const float* mix, const float* give,
+                    const float* take, const int32_t* rows, const float* weight, float eps, int rms, void* out, int dtype,
+                    int n_rows, int streams, int width, int write_x, hipStream_t stream);
+
+// gate_up[t] = [gate (width) | up (width)] in float32: g = min(gate, limit), u = clamp(up, -limit, limit),
+// out[t] = g * sigmoid(slope * g) * (u + 1) in `dtype`.
+int mll_clamped_glu(const float* gate_up, void* out, int dtype, int n_tokens, int width, float limit, float slope,
+                    hipStream_t stream);
+
+// ---- attention with a bias by distance and a sink, keys and values of different widths in plain pages --------
+
+// qkv[t] = [q (heads * key_dim) | k (kv_heads * key_dim) | v (kv_heads * value_dim)] in float32, perhaps in
+// n_parts parts that are added in order. Queries and keys are divided by their root mean square over their head
+// (+ eps inside the root) and multiplied by q_weight / k_weight [key_dim] (both null: no norm); queries are then
+// multiplied by 1 + temp_coef * ln((p + 1) / temp_every + 1) (whole-number division) at position p
+// (temp_coef 0: not). Queries go to q_out [t][heads][key_dim]; keys and values into the pages
+// [slot][kv_head][dim] at slot_mapping[t] (negative: not stored).
+int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
+                      float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
+                      void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
+                      int value_dim, hipStream_t stream);
+
+// Causal attention of every token over its request's pages: score_j = (q . k_j) * scale + bias[min(p - j, longest)][head]
+// (bias null: none; float32 [longest + 1][heads]); softmax over j <= p with exp(sink[head]) added to the denominator
+// (sink null: not); out[t][head] = out_scale * sum_j weight_j v_j, rows out_stride elements apart.
+// A token whose seq_of_token is negative is skipped. The order of every sum depends on p alone.
+int mll_bias_attention(const void* q, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_width,
+                       const int32_t* seq_of_token, const int32_t* positions, const float* bias, int longest,
+                       const float* sink, void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int kv_heads,
+                       int key_dim, int value_dim, int page_size, float scale, float out_scale, hipStream_t stream);
+
+// ---- gated linear attention --------------------------------------------------------------------------------
+
+// decay[t][c] = sigmoid(z)^(1 / tau), z = bias[c] + sum_r a2[c][r] * proj[t][low_offset + r]; float32 but a2.
+int mll_gla_decay(const float* proj, int64_t proj_stride, int low_offset, int rank, const void* a2, int a2_dtype,
+                  const float* bias, float tau, float* decay, int n_tokens, int channels, hipStream_t stream);
+
+// For every request i of the step, its tokens cu_tokens[i] .. cu_tokens[i + 1] - 1 in order, per head:
+//   S = diag(decay_t) S + k_t v_t^T;  out[t][head] = S^T (q_t * q_scale)
+// with S = state[slots[i]][head] (float32 [key_dim][value_dim]) read at the start and written at the end.
+// q, k, v are float32 columns of proj's rows at the given offsets. A request without tokens is passed over.
+int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset, const float* decay,
+                 float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
+                 int value_dim, float q_scale, hipStream_t stream);
+
+// out[t][head] = o[t][head] / rms(o[t][head]) * weight * silu(gate[t][head]) * out_scale, gate at gate_offset of
+// proj's rows; out in `dtype`, rows out_stride elements apart.
+int mll_gla_gate(const float* o, const float* proj, int64_t proj_stride, int gate_offset, const float* weight, float eps,
+                 void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int value_dim, float out_scale,
+                 hipStream_t stream);
+
 }  // extern "C"

@@ -12,6 +12,7 @@ from typing import Dict
 import numpy as np
 import torch
 
+from ..cache.needs import flat_bindings
 from ..parts.linear import Weight
 from ..sampling import Sampler, SamplingParams
 from .batch import StepEntry
@@ -19,8 +20,8 @@ from .engine import Engine
 
 
 def _fill_random(engine: Engine) -> None:
-    for binding in engine.cache.bindings():
-        if binding is not None and binding.need.paged and binding.owned:
+    for binding in (inner for binding in engine.cache.bindings() for inner in flat_bindings(binding)):
+        if binding.need.paged and binding.owned:
             for tensor in binding.tensors():
                 tensor.normal_(0.0, 1.0)
 

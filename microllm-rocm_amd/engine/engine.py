@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache, pages_of_group
+from ..cache.needs import flat_needs
 from ..cache.pages import OutOfPages
 from ..config.registry import architecture_named, load_config
 from ..ops import kernels, library
@@ -145,9 +146,12 @@ class Engine:
         del tensors, placed
         reads = [entry.reads_cache_of for entry in spec.order]
         self.max_portion = max_portion
-        self.cache = CacheManager(self.model.cache_needs(), reads, page_size, num_pages, max_requests,
-                                  dtype=self.dtype, device=self.device,
-                                  max_blocks=-(-spec.max_positions // page_size), max_portion=max_portion)
+        needs = self.model.cache_needs()
+        max_blocks = -(-spec.max_positions // page_size)
+        if all(inner.window is None for need in needs for inner in flat_needs(need)):
+            max_blocks = min(max_blocks, num_pages)     # without a window a request never holds more blocks than the pool has
+        self.cache = CacheManager(needs, reads, page_size, num_pages, max_requests, dtype=self.dtype, device=self.device,
+                                  max_blocks=max_blocks, max_portion=max_portion)
         self._bindings = self.cache.bindings()
         self._builder = BatchBuilder(self.cache, self.device, self.model.step_planners())
         self.steps_run = 0
@@ -175,9 +179,7 @@ class Engine:
             return True     # a float32 engine has no packed copies
         weights = sum(2 * int(torch.Size(decl.shape).numel()) for decl in decls.values())
         cache = 0
-        for need in model.cache_needs():
-            if need is None:
-                continue
+        for need in (inner for need in model.cache_needs() for inner in flat_needs(need)):
             if need.paged:
                 cache += pages_of_group(need, num_pages, page_size, max_requests, max_portion) * page_size * need.bytes_per_position(self.dtype)
             else:
@@ -326,7 +328,9 @@ class Engine:
     def _capture(self, state: "_DecodeGraph", ctx: StepContext) -> None:
         """Once eagerly (libraries create their handles and workspaces), then the capture. The step writes the same
         keys and values to the same slots each time, so running it again changes nothing."""
+        saved = self.cache.save_slots(ctx.host_slots)      # state in slots is not keys in pages: a second run would count
         self.model.forward(ctx, self._bindings, ctx.want_rows)
+        self.cache.restore_slots(saved)
         torch.cuda.synchronize(self.device)
         ctx.memo.clear()     # what the parts computed once for the step is computed inside the graph too
         if self._graph_pool is None:
@@ -443,9 +447,20 @@ class Engine:
 
         def after_entry(index, h, pending):
             stream = h.clone()
+            mix = give = None
+            if hasattr(pending, "values") and hasattr(pending, "give"):     # a delta for several streams (parts.streams)
+                pending, mix, give = pending.values, pending.mix, pending.give
             if isinstance(pending, torch.Tensor):   # else the entry's last product added its result itself
-                for part in (pending if pending.dim() == 3 else pending.unsqueeze(0)):
-                    stream += part.to(torch.float32)
+                delta = pending.to(torch.float32)
+                delta = delta.sum(0) if delta.dim() == 3 else delta
+                if stream.dim() == 3:
+                    if mix is not None:
+                        stream = torch.einsum("nsw,st->ntw", stream, mix)
+                    stream = stream + (give if give is not None else torch.ones_like(stream[0, :, 0]))[None, :, None] * delta[:, None, :]
+                else:
+                    stream += delta
+            if stream.dim() == 3:       # what a model of several streams hands on is their sum
+                stream = stream.sum(1)
             observer(index, stream)
 
         self.model.observer = after_entry

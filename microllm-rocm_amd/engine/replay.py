@@ -76,7 +76,7 @@ def main(argv=None) -> int:
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time; the cache pool is made for this many")
     parser.add_argument("--page-size", type=int, default=16)
-    parser.add_argument("--max-requests", type=int, default=16)
+    parser.add_argument("--max-requests", type=int, default=4, help="state slots: the most requests that are live at a time")
     parser.add_argument("--device", default="cuda:0")
     parser.add_argument("--dump-layers", action="store_true",
                         help="also write <step>.layers.f32: the residual stream at the wanted places after every layer")

@@ -978,3 +978,241 @@ def measured_peaks(device: Optional[torch.device] = None, read_bytes: int = 4 <<
     flops = blocks * 4 * iterations * 16 * 16384.0
     del data
     return {"hbm_read_GBps": round(read_bytes / read_time / 1e9, 1), "mfma_bf16_TFLOPs": round(flops / mfma_time / 1e12, 1)}
+
+
+# ---- several copies of the residual stream; a norm with a mean; a sinusoidal position vector --------------------
+def embedding_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, base: float) -> torch.Tensor:
+    """``table[ids] + wave(positions)`` in float32; entry 2i of the wave is ``sin(p * base^(-2i / width))``, entry
+    2i + 1 the cosine of the same angle."""
+    lib = library.load()
+    _device_tensor(table, "embedding table")
+    _device_tensor(ids, "token ids", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    _need(table.dim() == 2 and ids.dim() == 1 and positions.shape == ids.shape,
+          "embedding_sinusoid takes a [vocab, width] table and [tokens] ids and positions")
+    vocab, width = table.shape
+    out = torch.empty((ids.shape[0], width), dtype=torch.float32, device=table.device)
+    _check(lib.mll_embedding_sinusoid(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(positions), _ptr(out),
+                                      ids.shape[0], width, vocab, ctypes.c_double(base), _stream()), lib)
+    return out
+
+
+def stream_copies(h: torch.Tensor, copies: int) -> torch.Tensor:
+    """``[tokens, width]`` -> ``[tokens, copies, width]``, every copy equal to the row."""
+    lib = library.load()
+    _device_tensor(h, "stream", torch.float32)
+    _need(h.dim() == 2 and copies >= 1, "stream_copies takes [tokens, width] and a positive number of copies")
+    out = torch.empty((h.shape[0], copies, h.shape[1]), dtype=torch.float32, device=h.device)
+    _check(lib.mll_stream_copies(_ptr(h), _ptr(out), h.shape[0], h.shape[1], copies, _stream()), lib)
+    return out
+
+
+MAX_STREAMS = 8
+
+
+def stream_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, rms: bool = False,
+                delta: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                give: Optional[torch.Tensor] = None, take: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None, write_x: bool = False, want_out: bool = True) -> Optional[torch.Tensor]:
+    """The write of one sublayer's result into the streams, the read for the next and the norm between them.
+
+    ``x``: float32 ``[tokens, streams, width]`` (or ``[tokens, width]``: one stream). With ``delta`` (float32
+    ``[tokens, width]`` or parts ``[parts, tokens, width]``, added in order): ``x'_t = sum_s mix[s, t] x_s + give[t]
+    delta`` (``mix`` None: the identity, ``give`` None: ones), written back with ``write_x``. Then
+    ``u = sum_t take[t] x'_t`` (None: ones) and the result ``(u - mean) / sqrt(var + eps) * weight`` (``rms``:
+    ``u / sqrt(mean(u^2) + eps) * weight``) for the rows asked for; ``want_out`` False only writes the streams."""
+    lib = library.load()
+    _device_tensor(x, "streams", torch.float32)
+    _need(x.dim() in (2, 3), "streams are [tokens, streams, width] or [tokens, width]")
+    streams = x.shape[1] if x.dim() == 3 else 1
+    width = x.shape[-1]
+    _need(1 <= streams <= MAX_STREAMS, f"between 1 and {MAX_STREAMS} streams")
+    n_parts, part_stride = 1, 0
+    if delta is not None:
+        _device_tensor(delta, "delta", torch.float32)
+        if delta.dim() == 3:
+            n_parts, part_stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+            _need(n_parts >= 1 and tuple(delta.shape[1:]) == (x.shape[0], width), "delta parts must be [parts, tokens, width]")
+        else:
+            _need(tuple(delta.shape) == (x.shape[0], width), "delta must be [tokens, width]")
+    else:
+        _need(mix is None and give is None and not write_x, "without a delta there is nothing to write")
+    for name, tensor, shape in (("mix", mix, (streams, streams)), ("give", give, (streams,)), ("take", take, (streams,))):
+        if tensor is not None:
+            _device_tensor(tensor, name, torch.float32)
+            _need(tuple(tensor.shape) == shape, f"{name} must have shape {shape}")
+    if rows is not None:
+        _device_tensor(rows, "row selection", torch.int32)
+        _need(not write_x, "cannot write the streams through a row selection")
+        n_rows = rows.shape[0]
+    else:
+        n_rows = x.shape[0]
+    out = None
+    if want_out:
+        _need(weight is not None, "a norm needs its weight")
+        _device_tensor(weight, "norm weight", torch.float32)
+        _need(tuple(weight.shape) == (width,), "the norm weight must match the width")
+        out = torch.empty((n_rows, width), dtype=out_dtype, device=x.device)
+    _check(lib.mll_stream_norm(_ptr(x), _ptr(delta), n_parts, ctypes.c_int64(part_stride), _ptr(mix), _ptr(give), _ptr(take),
+                               _ptr(rows), _ptr(weight), ctypes.c_float(eps), int(rms), _ptr(out), _code(out_dtype),
+                               n_rows, streams, width, int(write_x), _stream()), lib)
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, slope: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``g * sigmoid(slope * g) * (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)`` of float32
+    rows ``[tokens, 2 * width]`` (gate first)."""
+    lib = library.load()
+    _device_tensor(gate_up, "gate/up", torch.float32)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate/up must be [tokens, 2 * width]")
+    n_tokens, width = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((n_tokens, width), dtype=out_dtype, device=gate_up.device)
+    for start in range(0, n_tokens, 65535):
+        count = min(65535, n_tokens - start)
+        _check(lib.mll_clamped_glu(ctypes.c_void_p(gate_up.data_ptr() + start * 2 * width * 4),
+                                   ctypes.c_void_p(out.data_ptr() + start * width * out.element_size()), _code(out_dtype),
+                                   count, width, ctypes.c_float(limit), ctypes.c_float(slope), _stream()), lib)
+    return out
+
+
+# ---- attention with a bias by distance and a sink ----------------------------------------------------------------
+def _parts_of(tensor: torch.Tensor, name: str) -> Tuple[int, int]:
+    _device_tensor(tensor, name, torch.float32)
+    _need(tensor.dim() in (2, 3), f"{name} must be [tokens, columns] or [parts, tokens, columns]")
+    if tensor.dim() == 3:
+        return tensor.shape[0], tensor.shape[1] * tensor.shape[2]
+    return 1, 0
+
+
+def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                  positions: torch.Tensor, slot_mapping: torch.Tensor, temp_coef: float, temp_every: int,
+                  k_pages: torch.Tensor, v_pages: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """Norm of queries and keys over their head, the queries' factor by position, keys and values into their pages
+    (``[page, position, kv_head, dim]``); returns the queries ``[tokens, heads * key_dim]``."""
+    lib = library.load()
+    n_parts, part_stride = _parts_of(qkv, "q/k/v")
+    n_tokens = qkv.shape[-2]
+    _need(qkv.shape[-1] == (heads + kv_heads) * key_dim + kv_heads * value_dim, "q/k/v rows have the wrong width")
+    _device_tensor(positions, "positions", torch.int32)
+    _device_tensor(slot_mapping, "slot mapping", torch.int32)
+    _need(positions.shape[0] >= n_tokens and slot_mapping.shape[0] >= n_tokens, "positions and slots for every token")
+    for name, weight in (("query norm weight", q_weight), ("key norm weight", k_weight)):
+        if weight is not None:
+            _device_tensor(weight, name, torch.float32)
+            _need(tuple(weight.shape) == (key_dim,), f"{name} must have the head's size")
+    _device_tensor(k_pages, "key pages", out_dtype)
+    _device_tensor(v_pages, "value pages", out_dtype)
+    _need(k_pages.dim() == 4 and tuple(k_pages.shape[2:]) == (kv_heads, key_dim), "key pages are [page, position, kv_head, key_dim]")
+    _need(v_pages.dim() == 4 and tuple(v_pages.shape[2:]) == (kv_heads, value_dim) and v_pages.shape[:2] == k_pages.shape[:2],
+          "value pages are [page, position, kv_head, value_dim]")
+    q_out = torch.empty((n_tokens, heads * key_dim), dtype=out_dtype, device=qkv.device)
+    _check(lib.mll_qk_norm_store(_ptr(qkv), n_parts, ctypes.c_int64(part_stride), _ptr(q_weight), _ptr(k_weight),
+                                 ctypes.c_float(eps), _ptr(positions), _ptr(slot_mapping), ctypes.c_float(temp_coef),
+                                 int(temp_every), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _code(out_dtype), n_tokens,
+                                 heads, kv_heads, key_dim, value_dim, _stream()), lib)
+    return q_out
+
+
+def bias_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                   seq_of_token: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor],
+                   sink: Optional[torch.Tensor], scale: float, out_scale: float, heads: int, kv_heads: int, key_dim: int,
+                   value_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention with ``bias[min(distance, last row), head]`` added to the scaled scores and ``exp(sink[head])``
+    in the softmax's denominator; ``out`` may be columns of a wider buffer (its row stride is taken)."""
+    lib = library.load()
+    _device_tensor(q, "queries")
+    n_tokens = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == heads * key_dim, "queries are [tokens, heads * key_dim]")
+    _device_tensor(k_pages, "key pages", q.dtype)
+    _device_tensor(v_pages, "value pages", q.dtype)
+    _need(k_pages.dim() == 4 and tuple(k_pages.shape[2:]) == (kv_heads, key_dim), "key pages are [page, position, kv_head, key_dim]")
+    _need(v_pages.dim() == 4 and tuple(v_pages.shape[2:]) == (kv_heads, value_dim) and v_pages.shape[:2] == k_pages.shape[:2],
+          "value pages are [page, position, kv_head, value_dim]")
+    page_size = k_pages.shape[1]
+    _device_tensor(block_table, "block table", torch.int32)
+    _device_tensor(seq_of_token, "request of every token", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    _need(block_table.dim() == 2 and seq_of_token.shape[0] >= n_tokens and positions.shape[0] >= n_tokens,
+          "a block table [requests, width] and a request and a position for every token")
+    longest = 0
+    if bias is not None:
+        _device_tensor(bias, "bias by distance", torch.float32)
+        _need(bias.dim() == 2 and bias.shape[1] == heads and bias.shape[0] >= 1, "the bias is [distances, heads]")
+        longest = bias.shape[0] - 1
+    if sink is not None:
+        _device_tensor(sink, "sink", torch.float32)
+        _need(tuple(sink.shape) == (heads,), "one sink a head")
+    if out is None:
+        out = torch.empty((n_tokens, heads * value_dim), dtype=q.dtype, device=q.device)
+    _need(out.is_cuda and out.dtype == q.dtype and out.dim() == 2 and tuple(out.shape) == (n_tokens, heads * value_dim)
+          and out.stride(1) == 1, "the output is [tokens, heads * value_dim] with unit column stride")
+    _check(lib.mll_bias_attention(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
+                                  _ptr(seq_of_token), _ptr(positions), _ptr(bias), longest, _ptr(sink),
+                                  ctypes.c_void_p(out.data_ptr()), ctypes.c_int64(out.stride(0) if n_tokens > 1 else max(out.stride(0), heads * value_dim)),
+                                  _code(q.dtype), n_tokens, heads, kv_heads, key_dim, value_dim, page_size,
+                                  ctypes.c_float(scale), ctypes.c_float(out_scale), _stream()), lib)
+    return out
+
+
+# ---- gated linear attention -----------------------------------------------------------------------------------
+def gla_decay(proj: torch.Tensor, low_offset: int, a2: torch.Tensor, bias: Optional[torch.Tensor], tau: float) -> torch.Tensor:
+    """``sigmoid(a2 @ low + bias)^(1 / tau)`` per token and key channel, ``low`` being columns of ``proj``'s rows."""
+    lib = library.load()
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(a2, "decay weight")
+    _need(proj.dim() == 2 and a2.dim() == 2, "projections [tokens, columns] and a decay weight [channels, rank]")
+    channels, rank = a2.shape
+    if bias is not None:
+        _device_tensor(bias, "decay bias", torch.float32)
+        _need(tuple(bias.shape) == (channels,), "one bias a channel")
+    n_tokens = proj.shape[0]
+    decay = torch.empty((n_tokens, channels), dtype=torch.float32, device=proj.device)
+    for start in range(0, n_tokens, 65535):
+        count = min(65535, n_tokens - start)
+        _check(lib.mll_gla_decay(ctypes.c_void_p(proj.data_ptr() + start * proj.shape[1] * 4), ctypes.c_int64(proj.shape[1]),
+                                 low_offset, rank, _ptr(a2), _code(a2.dtype), _ptr(bias), ctypes.c_float(tau),
+                                 ctypes.c_void_p(decay.data_ptr() + start * channels * 4), count, channels, _stream()), lib)
+    return decay
+
+
+def gla_scan(proj: torch.Tensor, q_offset: int, k_offset: int, v_offset: int, decay: torch.Tensor, state: torch.Tensor,
+             cu_tokens: torch.Tensor, slots: torch.Tensor, n_seqs: int, heads: int, key_dim: int, value_dim: int,
+             q_scale: float) -> torch.Tensor:
+    """The recurrence over every request's tokens of the step; ``state`` is ``[slots, heads, key_dim, value_dim]``
+    float32, read and written at ``slots``. Returns ``[tokens, heads * value_dim]`` float32."""
+    lib = library.load()
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(decay, "decays", torch.float32)
+    _device_tensor(state, "state", torch.float32)
+    _device_tensor(cu_tokens, "token offsets", torch.int32)
+    _device_tensor(slots, "state slots", torch.int32)
+    n_tokens = proj.shape[0]
+    _need(proj.dim() == 2 and tuple(decay.shape) == (n_tokens, heads * key_dim), "decays are [tokens, heads * key_dim]")
+    _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, key_dim, value_dim), "state is [slots, heads, key_dim, value_dim]")
+    _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
+    out = torch.empty((n_tokens, heads * value_dim), dtype=torch.float32, device=proj.device)
+    _check(lib.mll_gla_scan(_ptr(proj), ctypes.c_int64(proj.shape[1]), q_offset, k_offset, v_offset, _ptr(decay), _ptr(state),
+                            _ptr(cu_tokens), _ptr(slots), _ptr(out), n_seqs, heads, key_dim, value_dim,
+                            ctypes.c_float(q_scale), _stream()), lib)
+    return out
+
+
+def gla_gate(o: torch.Tensor, proj: torch.Tensor, gate_offset: int, weight: torch.Tensor, eps: float, heads: int,
+             value_dim: int, out_scale: float, out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per head: ``o / rms(o) * weight * silu(gate) * out_scale``; ``out`` may be columns of a wider buffer."""
+    lib = library.load()
+    _device_tensor(o, "recurrence output", torch.float32)
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(weight, "norm weight", torch.float32)
+    n_tokens = o.shape[0]
+    _need(tuple(o.shape) == (n_tokens, heads * value_dim) and proj.shape[0] == n_tokens and tuple(weight.shape) == (value_dim,),
+          "gla_gate takes [tokens, heads * value_dim], the projections of the same tokens and a weight [value_dim]")
+    if out is None:
+        out = torch.empty((n_tokens, heads * value_dim), dtype=out_dtype, device=o.device)
+    _need(out.is_cuda and out.dtype == out_dtype and tuple(out.shape) == (n_tokens, heads * value_dim) and out.stride(1) == 1,
+          "the output is [tokens, heads * value_dim] with unit column stride")
+    _check(lib.mll_gla_gate(_ptr(o), _ptr(proj), ctypes.c_int64(proj.shape[1]), gate_offset, _ptr(weight), ctypes.c_float(eps),
+                            ctypes.c_void_p(out.data_ptr()), ctypes.c_int64(max(out.stride(0), heads * value_dim)), _code(out_dtype),
+                            n_tokens, heads, value_dim, ctypes.c_float(out_scale), _stream()), lib)
+    return out

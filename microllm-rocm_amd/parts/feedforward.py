@@ -56,3 +56,40 @@ class SwiGLU(FeedForward):
 
 
 register_part("ffn", "swiglu", SwiGLU)
+
+
+class ClampedGLU(FeedForward):
+    """A gated feed-forward with clamped inputs: ``g = min(gate(x), limit)``, ``u = clamp(up(x), -limit, limit)``,
+    ``down(g * sigmoid(slope * g) * (u + 1))``, no biases. Gate and up are one stacked product whose float32 result
+    the activation rounds once."""
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        self.hidden = int(spec.params["hidden_size"])
+        self.intermediate = int(spec.params["intermediate_size"])
+        self.limit = float(spec.params["limit"])
+        self.slope = float(spec.params.get("slope", 1.702))
+        self.gate_up_weight: Optional[Weight] = None
+        self.down_weight: Optional[Weight] = None
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        return {self.name("gate"): TensorDecl((self.intermediate, self.hidden), MATRIX),
+                self.name("up"): TensorDecl((self.intermediate, self.hidden), MATRIX),
+                self.name("down"): TensorDecl((self.hidden, self.intermediate), MATRIX)}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        gate, up = tensors[self.name("gate")], tensors[self.name("up")]
+        if gate.dtype != up.dtype:
+            raise TypeError("the gate and up weights of one layer must share a dtype to be stacked")
+        self.gate_up_weight = Weight(torch.cat([gate, up], dim=0).contiguous(), keep_plain=self.runtime.keep_plain_weights)
+        del gate, up
+        self.down_weight = Weight(tensors[self.name("down")], keep_plain=self.runtime.keep_plain_weights)
+
+    def forward(self, x, ctx):
+        gate_up = linear(x, self.gate_up_weight, out_dtype=torch.float32)
+        z = kernels.clamped_glu(gate_up, self.limit, self.slope, self.runtime.dtype)
+        return linear(z, self.down_weight, out_dtype=torch.float32, partials=True)
+
+
+register_part("ffn", "clamped_glu", ClampedGLU)

@@ -174,6 +174,8 @@ class Model:
         ``want_rows`` indexes the step's flat token list; None or empty skips the head.
         """
         h = self.embedding.forward(ctx)
+        if self.spec.streams is not None:       # every copy starts as the embedding's output
+            h = kernels.stream_copies(h, self.spec.streams)
         pending = None
         order = self.spec.order
         for index, entry in enumerate(order):

@@ -60,6 +60,7 @@ class ModelSpec:
     order: Tuple[RunEntry, ...]
     final_norm: PartSpec
     head: PartSpec
+    streams: Optional[int] = None   # copies of the residual stream (``parts.streams``); None: one, held as [tokens, hidden]
 
     def validate(self) -> None:
         if not self.layers or not self.order:

@@ -199,3 +199,17 @@ def open_model_files(folder: str) -> Tuple[Dict[str, SafetensorsFile], Dict[str,
                 raise SafetensorsError(f"tensor {name!r} is in both {owner[name]} and {file_name}")
             owner[name] = file_name
     return files, owner
+
+
+def tensor_shapes(folder: str) -> Dict[str, Tuple[int, ...]]:
+    """Name -> shape of every tensor in a model folder, read from the headers alone; empty if the folder holds no
+    tensor files (a configuration may be read before its weights are written)."""
+    try:
+        files, owner = open_model_files(folder)
+    except FileNotFoundError:
+        return {}
+    try:
+        return {name: tuple(files[file_name].entries[name].shape) for name, file_name in owner.items()}
+    finally:
+        for handle in files.values():
+            handle.close()
