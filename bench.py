@@ -59,6 +59,76 @@ def serve(args, config, full_layers: int, page_size: int) -> int:
     return 0
 
 
+DESIGN_SIZES = {
+    # width, query heads, kv heads, head size, feed-forward width, layers; the linear attention beside the softmax
+    # attention of a Siditar layer has half as many heads, keys of half the head size and values of the whole
+    "1k": dict(width=1024, heads=8, kv_heads=2, head_dim=128, ff=4096, layers=4),
+    "2k": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ff=8192, layers=4),
+    "4k": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=14336, layers=2),
+}
+DESIGN_VOCAB = 32768
+
+
+def design_configs(size: dict):
+    """A Siditar configuration of the given layer sizes and the Qwen2 configuration of equal width, heads, head size,
+    feed-forward width, depth and vocabulary."""
+    from microllm_rocm_amd import Qwen2Config
+    from microllm_rocm_amd.config.siditar import (BiasAttentionConfig, DenseMlpConfig, LinearAttentionConfig,
+                                                  ParallelMixerConfig, SiditarConfig, SiditarLayerConfig)
+    left = BiasAttentionConfig(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["head_dim"], vdim=size["head_dim"],
+                               scale=size["head_dim"] ** -0.5, bias_max=1024, temp_coef=0.5, temp_every=64, bias_rows=32)
+    right = LinearAttentionConfig(heads=size["heads"] // 2, dim=size["head_dim"] // 2, vdim=size["head_dim"], tau=16.0, decay_rank=16)
+    layer = SiditarLayerConfig("parallel", ParallelMixerConfig(left, right, 1.0, 1.0), DenseMlpConfig(size["ff"], 7.0))
+    siditar = SiditarConfig(vocab=DESIGN_VOCAB, width=size["width"], norm_eps=1e-6, layers=(layer,) * size["layers"], streams=2)
+    qwen2 = Qwen2Config(vocab_size=DESIGN_VOCAB, hidden_size=size["width"], num_hidden_layers=size["layers"],
+                        num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["head_dim"],
+                        intermediate_size=size["ff"], max_position_embeddings=32768, rope_theta=1e6, rms_norm_eps=1e-6,
+                        tie_word_embeddings=False)
+    return {"siditar": siditar, "qwen2": qwen2}
+
+
+def compare_designs(args) -> int:
+    """Prefill and decode throughput of the Siditar design beside Qwen2 at equal layer sizes; prints one JSON line."""
+    import torch
+    from microllm_rocm_amd import Engine
+    from microllm_rocm_amd.engine.benchmark import decode_throughput, prefill_throughput, step_bytes, step_flops
+    page_size, rows = 16, []
+    peak_flops = BF16_PEAK_FLOPS if args.dtype == "bfloat16" else FP32_PEAK_FLOPS
+    for name in [part for part in args.design_sizes.split(",") if part]:
+        size = DESIGN_SIZES[name]
+        for design, config in design_configs(size).items():
+            if args.design_only and design != args.design_only:
+                continue
+            per_request = args.context + args.steps + args.warmup + 2 * page_size
+            engine = Engine.from_random(config, seed=0, dtype=args.dtype, device="cuda:0", on_device=True, page_size=page_size,
+                                        max_tokens=max(args.batch * per_request, args.prefill_tokens + page_size),
+                                        max_requests=max(args.batch, 4))
+            row = {"design": design, "size": name, **size}
+            if not args.no_prefill:
+                prefill = prefill_throughput(engine, args.prefill_tokens, repeats=3)
+                flops = step_flops(engine, args.prefill_tokens)
+                row["prefill"] = {"tokens": args.prefill_tokens, "tok_per_s": round(prefill["tokens_per_second"], 1),
+                                  "ms": round(prefill["ms"], 3), "frac_of_peak": round(flops / (prefill["ms"] * 1e-3) / peak_flops, 4)}
+            decode = decode_throughput(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
+            moved = step_bytes(engine, args.batch, args.context + args.warmup + args.steps // 2)
+            row["decode"] = {"batch": args.batch, "context": args.context, "tok_per_s": round(decode["tokens_per_second"], 1),
+                             "ms_per_step": round(decode["ms_per_step"], 4),
+                             "frac_of_hbm": round(moved / (decode["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            rows.append(row)
+            del engine
+            torch.cuda.empty_cache()
+    first = next((row for row in rows if row["design"] == "siditar"), rows[0])
+    line = {"metric": "decode tok/s of the Siditar design beside Qwen2 at equal layer sizes", "value": first["decode"]["tok_per_s"],
+            "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["decode"]["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: random weights, uniform-random token ids, caches filled with random keys and values",
+            "config": {"model": f"Siditar and Qwen2 at sizes {args.design_sizes}", "global_batch": args.batch, "seq_len": args.context,
+                       "vocab": DESIGN_VOCAB, "kv_block_size": page_size, "parallelism": "single GPU"},
+            "compare": rows}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -85,6 +155,11 @@ def main() -> int:
     parser.add_argument("--no-extras", action="store_true",
                         help="leave out what the default run adds to its line after the main figures: decoding on the 32-bit path "
                              "at batch 8 and the continuous-batching workload at Qwen2-0.5B sizes")
+    parser.add_argument("--design", default=None, choices=["siditar"],
+                        help="instead of the default workload: prefill and decode throughput of this design beside Qwen2 at equal "
+                             "layer sizes (--design-sizes), random weights; --batch, --context, --prefill-tokens, --steps apply")
+    parser.add_argument("--design-sizes", default="1k,2k,4k", help="of " + ", ".join(sorted(DESIGN_SIZES)))
+    parser.add_argument("--design-only", default=None, choices=["siditar", "qwen2"], help="one of the two designs alone (profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
@@ -94,6 +169,8 @@ def main() -> int:
     from microllm_rocm_amd import Engine, Qwen2Config
     from microllm_rocm_amd.engine.benchmark import decode_throughput, prefill_throughput, step_bytes, step_flops
 
+    if args.design:
+        return compare_designs(args)
     sizes = dict(SIZES[args.size])
     full_layers = sizes.pop("num_hidden_layers")
     if args.layers is None:

@@ -10,6 +10,7 @@
 // of one key, the tile's maximum and weights follow, and then the lanes turn to the value's channels and add the
 // 64 weighted values in key order. The order of every sum depends on the query's position alone, so a row does
 // not change with the step's cut, the batch or the pages. Scores, weights and sums are float32.
+#include "cache_layout.h"
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -128,7 +129,8 @@ __global__ void __launch_bounds__(kWave)
 qk_norm_store_kernel(const float* __restrict__ qkv, int n_parts, int64_t part_stride, const float* __restrict__ q_weight,
                      const float* __restrict__ k_weight, float eps, const int32_t* __restrict__ positions,
                      const int32_t* __restrict__ slot_mapping, float temp_coef, int temp_every, T* __restrict__ q_out,
-                     T* __restrict__ k_pages, T* __restrict__ v_pages, int heads, int kv_heads, int key_dim, int value_dim) {
+                     T* __restrict__ k_pages, T* __restrict__ v_pages, int heads, int kv_heads, int key_dim, int value_dim,
+                     int tiled_page_size) {
     const int vectors = heads + 2 * kv_heads;
     const int token = blockIdx.x / vectors;
     const int which = blockIdx.x % vectors;
@@ -157,10 +159,21 @@ qk_norm_store_kernel(const float* __restrict__ qkv, int n_parts, int64_t part_st
     T* to = is_q ? q_out + (static_cast<int64_t>(token) * heads + head) * key_dim
                  : (is_k ? k_pages + (static_cast<int64_t>(slot) * kv_heads + head) * key_dim
                          : v_pages + (static_cast<int64_t>(slot) * kv_heads + head) * value_dim);
+    // tiled_page_size > 0: the pages are in the order the MFMA kernels read them (cache_layout.h; both widths equal)
+    const bool tiled = tiled_page_size > 0 && !is_q;
+    const CacheLayout layout(kv_heads, tiled ? tiled_page_size : 16, key_dim);
+    const int64_t page = tiled ? slot / tiled_page_size : 0;
+    const int in_page = tiled ? slot % tiled_page_size : 0;
     for (int c = lane; c < dim; c += kWave) {
         float value = row[offset + c];
         for (int part = 1; part < n_parts; ++part) value += row[part * part_stride + offset + c];
-        to[c] = from_float<T>(weight ? value * factor * weight[c] : value);
+        const T rounded = from_float<T>(weight ? value * factor * weight[c] : value);
+        if (tiled) {
+            if (is_k) k_pages[layout.k_at(page, head, in_page, c)] = rounded;
+            else v_pages[layout.v_at(page, head, in_page, c)] = rounded;
+        } else {
+            to[c] = rounded;
+        }
     }
 }
 
@@ -173,7 +186,9 @@ extern "C" {
 int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
                       float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
                       void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, hipStream_t stream) {
+                      int value_dim, int tiled_page_size, hipStream_t stream) {
+    MLL_REQUIRE(tiled_page_size == 0 || (tiled_page_size > 0 && tiled_page_size % 16 == 0 && key_dim == value_dim),
+                "qk_norm_store: tiled pages hold a multiple of 16 positions and keys and values of one width");
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0, "qk_norm_store: sizes must be positive");
     MLL_REQUIRE(n_parts >= 1, "qk_norm_store: at least one part");
     MLL_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qk_norm_store: norm weights for queries and keys, or for neither");
@@ -185,11 +200,13 @@ int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const 
     if (dtype == kF32) {
         qk_norm_store_kernel<float><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
             qkv, n_parts, part_stride, q_weight, k_weight, eps, positions, slot_mapping, temp_coef, temp_every,
-            static_cast<float*>(q_out), static_cast<float*>(k_pages), static_cast<float*>(v_pages), heads, kv_heads, key_dim, value_dim);
+            static_cast<float*>(q_out), static_cast<float*>(k_pages), static_cast<float*>(v_pages), heads, kv_heads, key_dim, value_dim,
+            tiled_page_size);
     } else if (dtype == kBF16) {
         qk_norm_store_kernel<bf16><<<static_cast<unsigned>(blocks), kWave, 0, stream>>>(
             qkv, n_parts, part_stride, q_weight, k_weight, eps, positions, slot_mapping, temp_coef, temp_every,
-            static_cast<bf16*>(q_out), static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), heads, kv_heads, key_dim, value_dim);
+            static_cast<bf16*>(q_out), static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), heads, kv_heads, key_dim, value_dim,
+            tiled_page_size);
     } else {
         return fail("qk_norm_store: unknown dtype");
     }

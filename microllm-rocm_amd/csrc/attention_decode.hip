@@ -40,13 +40,16 @@ union Frag8 {
     uint4 raw;
 };
 
-template <int HD_TILES, bool STREAM>
+// EXTRA: the scores also get extras.bias[min(position - key, longest)][head], the softmax's denominator also holds
+// exp(extras.sink[head]) (counted once, where the waves' or the splits' results meet), the result is multiplied by
+// extras.out_scale and its rows lie extras.out_stride elements apart. Without EXTRA the kernel is what it was.
+template <int HD_TILES, bool STREAM, bool EXTRA>
 __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ token_ids, bf16* __restrict__ out,
     float* __restrict__ part_o, float* __restrict__ part_ml, float scale, int window, int heads, int kv_heads,
-    int page_size, int n_splits) {
+    int page_size, int n_splits, MllAttentionExtras extras) {
     constexpr int HD = HD_TILES * 16;
     constexpr int K_STEPS = (HD + 31) / 32;
     constexpr int K_CHUNKS = HD / 8;
@@ -100,6 +103,13 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
 #pragma unroll
     for (int d = 0; d < HD_TILES; ++d) o_acc[d] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float running_max = -INFINITY, running_sum = 0.0f;
+    // The bias of this lane's head: one column of the table; every distance from `longest` on has the last row's.
+    const float* bias_column = nullptr;
+    float far_bias = 0.0f;
+    if (EXTRA && extras.bias != nullptr) {
+        bias_column = extras.bias + head0 + min(col, heads_here - 1);
+        far_bias = bias_column[static_cast<int64_t>(extras.longest) * heads];
+    }
 
     // A pair's keys and values, from the pages into registers. A lane's 8 k-slots of the second product are the
     // 8 positions 8 * (quad % 2) .. + 7 of tile quad / 2 of the pair: one load of 16 bytes per 16 dims from the
@@ -149,7 +159,12 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = key0 + 8 * quad + 4 * t + i;
-                score[4 * t + i] = (key >= low && key <= position) ? s[i] * scale : -INFINITY;
+                float value = s[i] * scale;
+                if (EXTRA && bias_column != nullptr) {
+                    const int distance = position - key;
+                    value += (distance >= extras.longest || distance < 0) ? far_bias : bias_column[static_cast<int64_t>(distance) * heads];
+                }
+                score[4 * t + i] = (key >= low && key <= position) ? value : -INFINITY;
             }
         }
         // A pair that straddles an end of the visible range may hold stale values: they must not reach
@@ -268,6 +283,8 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
         float top = m_shared[0][h];
 #pragma unroll
         for (int w = 1; w < kSlots; ++w) top = fmaxf(top, m_shared[w][h]);
+        const bool sink_here = EXTRA && extras.sink != nullptr && n_splits == 1;      // else the join kernel counts it
+        if (sink_here) top = fmaxf(top, extras.sink[head0 + h]);
         float total = 0.0f, sum = 0.0f;
 #pragma unroll
         for (int w = 0; w < kSlots; ++w) {
@@ -276,10 +293,12 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
             total += weight * o_shared[w][h][dim];
             sum += weight * l_shared[w][h];
         }
+        if (sink_here) sum += __expf(extras.sink[head0 + h] - top);
         const int64_t row = static_cast<int64_t>(token) * heads + head0 + h;
         const int64_t part_row = static_cast<int64_t>(blockIdx.x) * heads + head0 + h;   // partial results are kept densely
         if (n_splits == 1) {
-            out[row * HD + dim] = from_float<bf16>(total / sum);
+            if (EXTRA) out[static_cast<int64_t>(token) * extras.out_stride + (head0 + h) * HD + dim] = from_float<bf16>(total / sum * extras.out_scale);
+            else out[row * HD + dim] = from_float<bf16>(total / sum);
         } else {
             part_o[(part_row * n_splits + split) * HD + dim] = total;
             if (dim == 0) {
@@ -291,9 +310,10 @@ __global__ __launch_bounds__(kDecodeThreads) void paged_attention_decode_kernel(
 }
 
 // Joins the splits of one (token, head): out = sum_s w_s O_s / sum_s w_s l_s with w_s = exp(m_s - max m).
+template <bool EXTRA>
 __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                             const int32_t* __restrict__ token_ids, bf16* __restrict__ out, int heads,
-                                            int head_dim, int n_splits) {
+                                            int head_dim, int n_splits, MllAttentionExtras extras) {
     const int token = token_ids ? token_ids[blockIdx.x / heads] : blockIdx.x / heads;
     if (token < 0) return;      // an entry that only pads the list to a fixed length
     const int64_t row = static_cast<int64_t>(token) * heads + blockIdx.x % heads;
@@ -308,6 +328,9 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
 #pragma unroll
         for (int j = 0; j < 8; ++j) top = fmaxf(top, pair[j].x);
     }
+    const bool with_sink = EXTRA && extras.sink != nullptr;
+    const float sink = with_sink ? extras.sink[blockIdx.x % heads] : 0.0f;
+    if (with_sink) top = fmaxf(top, sink);
     for (int dim = threadIdx.x; dim < head_dim; dim += blockDim.x) {
         float total = 0.0f, weight_sum = 0.0f;
         for (int base = 0; base < n_splits; base += 8) {
@@ -327,7 +350,9 @@ __global__ void paged_attention_join_kernel(const float* __restrict__ part_o, co
                 weight_sum += weight * pair[j].y;
             }
         }
-        out[row * head_dim + dim] = from_float<bf16>(total / weight_sum);
+        if (with_sink) weight_sum += __expf(sink - top);
+        if (EXTRA) out[static_cast<int64_t>(token) * extras.out_stride + (blockIdx.x % heads) * head_dim + dim] = from_float<bf16>(total / weight_sum * extras.out_scale);
+        else out[row * head_dim + dim] = from_float<bf16>(total / weight_sum);
     }
 }
 
@@ -335,16 +360,22 @@ template <int HD_TILES>
 static int launch_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                          int table_width, const int32_t* seq_of_token, const int32_t* positions,
                          const int32_t* token_ids, void* out, float* part_o, float* part_ml, float scale, int window,
-                         int n_tokens, int heads, int kv_heads, int page_size, int n_splits, hipStream_t stream) {
+                         int n_tokens, int heads, int kv_heads, int page_size, int n_splits, const MllAttentionExtras* extras,
+                         hipStream_t stream) {
     const int group = heads / kv_heads;
+    const MllAttentionExtras given = extras ? *extras : MllAttentionExtras{nullptr, 0, nullptr, 1.0f, 0};
     const dim3 grid(n_tokens, kv_heads * ((group + 15) / 16), n_splits);
     const bool stream_pages = static_cast<int64_t>(grid.x) * grid.y * grid.z >= 256;      // a workgroup per compute unit or more
-#define MLL_DECODE_LAUNCH(STREAM)                                                                                     \
-    paged_attention_decode_kernel<HD_TILES, STREAM><<<grid, kDecodeThreads, 0, stream>>>(                             \
+#define MLL_DECODE_LAUNCH(STREAM, EXTRA)                                                                              \
+    paged_attention_decode_kernel<HD_TILES, STREAM, EXTRA><<<grid, kDecodeThreads, 0, stream>>>(                      \
         static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table, \
         table_width, seq_of_token, positions, token_ids, static_cast<bf16*>(out), part_o, part_ml, scale, window, heads, \
-        kv_heads, page_size, n_splits)
-    if (stream_pages) MLL_DECODE_LAUNCH(true); else MLL_DECODE_LAUNCH(false);
+        kv_heads, page_size, n_splits, given)
+    if (extras) {
+        if (stream_pages) MLL_DECODE_LAUNCH(true, true); else MLL_DECODE_LAUNCH(false, true);
+    } else {
+        if (stream_pages) MLL_DECODE_LAUNCH(true, false); else MLL_DECODE_LAUNCH(false, false);
+    }
 #undef MLL_DECODE_LAUNCH
     return check_launch("paged_attention_decode");
 }
@@ -358,6 +389,19 @@ extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, co
                                           const int32_t* positions, const int32_t* token_ids, void* out, float* part_o,
                                           float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
                                           int head_dim, int page_size, int n_splits, hipStream_t stream) {
+    return mll_paged_attention_decode_extra(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions, token_ids,
+                                            out, part_o, part_ml, scale, window, n_tokens, heads, kv_heads, head_dim, page_size,
+                                            n_splits, nullptr, stream);
+}
+
+extern "C" int mll_paged_attention_decode_extra(const void* q, const void* k_cache, const void* v_cache,
+                                                const int32_t* block_table, int table_width, const int32_t* seq_of_token,
+                                                const int32_t* positions, const int32_t* token_ids, void* out, float* part_o,
+                                                float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
+                                                int head_dim, int page_size, int n_splits, const MllAttentionExtras* extras,
+                                                hipStream_t stream) {
+    MLL_REQUIRE(!extras || extras->out_stride >= static_cast<int64_t>(heads) * head_dim, "paged_attention_decode: the output rows overlap");
+    MLL_REQUIRE(!extras || !extras->bias || extras->longest >= 0, "paged_attention_decode: the bias table needs a row");
     MLL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "paged_attention_decode: heads must divide into kv_heads groups");
     MLL_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
                 "paged_attention_decode: head_dim must be a multiple of 16 in [16, 256]");
@@ -371,7 +415,7 @@ extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, co
     case TILES:                                                                                                       \
         status = launch_decode<TILES>(q, k_cache, v_cache, block_table, table_width, seq_of_token, positions,         \
                                       token_ids, out, part_o, part_ml, scale, window, n_tokens, heads, kv_heads,      \
-                                      page_size, n_splits, stream);                                                   \
+                                      page_size, n_splits, extras, stream);                                           \
         break;
     switch (head_dim / 16) {
         MLL_DECODE_CASE(1) MLL_DECODE_CASE(2) MLL_DECODE_CASE(3) MLL_DECODE_CASE(4) MLL_DECODE_CASE(5)
@@ -384,8 +428,13 @@ extern "C" int mll_paged_attention_decode(const void* q, const void* k_cache, co
     if (status != 0) return status;
     if (n_splits > 1) {
         const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
-        paged_attention_join_kernel<<<n_tokens * heads, threads, 0, stream>>>(part_o, part_ml, token_ids,
-                                                                             static_cast<bf16*>(out), heads, head_dim, n_splits);
+        if (extras) {
+            paged_attention_join_kernel<true><<<n_tokens * heads, threads, 0, stream>>>(part_o, part_ml, token_ids, static_cast<bf16*>(out),
+                                                                                       heads, head_dim, n_splits, *extras);
+        } else {
+            paged_attention_join_kernel<false><<<n_tokens * heads, threads, 0, stream>>>(part_o, part_ml, token_ids, static_cast<bf16*>(out),
+                                                                                        heads, head_dim, n_splits, MllAttentionExtras{nullptr, 0, nullptr, 1.0f, 0});
+        }
         return check_launch("paged_attention_join");
     }
     return 0;

@@ -55,12 +55,19 @@ __device__ inline float reduce_lanes_32_apart(float value, Op op) {
 }
 
 
-template <int HD_TILES>
+constexpr int kPrefillBiasRows = 4096;      // the longest bias table (one column of it is kept in LDS, 16 KB)
+
+// EXTRA: a bias by distance on the scores, a sink in the softmax, a factor on the result and a stride between its
+// rows (MllAttentionExtras). The bias column of the workgroup's head lies in LDS in the scores' own units (divided
+// by scale); a run of keys all of which lie `longest` or further behind all of the wave's tokens takes the last
+// row's value for every score, any other run looks every score's distance up. The sink is where the running
+// maximum and sum start. Without EXTRA the kernel is what it was.
+template <int HD_TILES, bool EXTRA>
 __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
     const int32_t* __restrict__ positions, bf16* __restrict__ out, float scale, int window, int heads,
-    int kv_heads, int page_size) {
+    int kv_heads, int page_size, MllAttentionExtras extras) {
     constexpr int HD = HD_TILES * 16;
     constexpr int K_STEPS = HD_TILES;                            // steps of 16 dims of the first product
     constexpr int D_BLOCKS = (HD + 31) / 32;                     // blocks of 32 dims of the second product's result
@@ -74,6 +81,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     // knows that a load into one stage does not write what is read from the other, and lets the two overlap.
     __shared__ __align__(16) bf16 stage_even[STAGE_ELEMENTS];
     __shared__ __align__(16) bf16 stage_odd[STAGE_ELEMENTS];
+    __shared__ float bias_column[EXTRA ? kPrefillBiasRows : 1];
 
     // Which entry and head this workgroup takes. Workgroups go to the GPU's 8 dies (each with a second-level cache
     // of its own) by turns, in the order of their number; numbered entry-first, every die would read every kv
@@ -166,6 +174,19 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
     float running_max = -INFINITY;
     float running_sum = 0.0f;         // over this lane's keys only; the two halves of the wave meet at the end
     float running_offset = 0.0f;      // -(running maximum) in units of log 2; 0 while the maximum is -inf
+    const bool biased = EXTRA && extras.bias != nullptr;
+    if (EXTRA) {
+        const float to_units = 1.0f / scale;
+        if (biased) {       // read after the first block has landed, which is behind a barrier
+            for (int row = threadIdx.x; row <= extras.longest; row += kPrefillThreads)
+                bias_column[row] = extras.bias[static_cast<int64_t>(row) * heads + head] * to_units;
+        }
+        if (extras.sink != nullptr) {      // one more term of every token's sum, of weight exp(sink - maximum)
+            running_max = extras.sink[head] * to_units;
+            running_offset = -running_max * scale_log2;
+            running_sum = half == 0 ? 1.0f : 0.0f;
+        }
+    }
 
     // Copy of one block's tiles, from the pages straight into LDS (no registers in between): a wave moves 64
     // consecutive pieces of 16 bytes of the block's key tiles as they lie in LDS, piece pass * threads + thread,
@@ -320,6 +341,23 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
             if (j + kAhead < PRODUCTS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         // s[r][i] is row 8 (i / 4) + 4 half + i % 4: key key0 + 32 r + 16 (i / 8) + 8 half + i % 8, token `column`.
+        if (EXTRA && biased) {
+            if (block_position - (key0 + 32 * HALVES - 1) >= extras.longest) {      // every key far behind every token
+                const float far = bias_column[extras.longest];
+#pragma unroll
+                for (int r = 0; r < HALVES; ++r)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) s[r][i] += far;
+            } else {
+#pragma unroll
+                for (int r = 0; r < HALVES; ++r)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int distance = my_position - (key0 + 32 * r + 16 * (i / 8) + 8 * half + (i % 8));
+                        s[r][i] += bias_column[min(max(distance, 0), extras.longest)];
+                    }
+            }
+        }
         if (MASKED) {
 #pragma unroll
             for (int r = 0; r < HALVES; ++r)
@@ -442,8 +480,9 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 
     // o_acc[d][i]: dim 32 d + 8 (i / 4) + 4 half + i % 4 of token `column`.
     if (column < block_valid) {
-        const float inverse = 1.0f / running_sum;
-        bf16* out_row = out + (static_cast<int64_t>(first_token + block_first + column) * heads + head) * HD;
+        const float inverse = (EXTRA ? extras.out_scale : 1.0f) / running_sum;
+        bf16* out_row = EXTRA ? out + static_cast<int64_t>(first_token + block_first + column) * extras.out_stride + head * HD
+                              : out + (static_cast<int64_t>(first_token + block_first + column) * heads + head) * HD;
 #pragma unroll
         for (int d = 0; d < D_BLOCKS; ++d)
 #pragma unroll
@@ -461,11 +500,19 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void paged_attention_prefill_ke
 template <int HD_TILES>
 static int launch_prefill(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                           int table_width, const int32_t* tiles, int n_tiles, const int32_t* positions, void* out,
-                          float scale, int window, int heads, int kv_heads, int page_size, hipStream_t stream) {
+                          float scale, int window, int heads, int kv_heads, int page_size, const MllAttentionExtras* extras,
+                          hipStream_t stream) {
     const dim3 grid(n_tiles, heads);   // n_tiles: workgroups, of two tiles each
-    paged_attention_prefill_kernel<HD_TILES><<<grid, kPrefillThreads, 0, stream>>>(
-        static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,
-        table_width, tiles, positions, static_cast<bf16*>(out), scale, window, heads, kv_heads, page_size);
+    if (extras) {
+        paged_attention_prefill_kernel<HD_TILES, true><<<grid, kPrefillThreads, 0, stream>>>(
+            static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,
+            table_width, tiles, positions, static_cast<bf16*>(out), scale, window, heads, kv_heads, page_size, *extras);
+    } else {
+        paged_attention_prefill_kernel<HD_TILES, false><<<grid, kPrefillThreads, 0, stream>>>(
+            static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache), static_cast<const bf16*>(v_cache), block_table,
+            table_width, tiles, positions, static_cast<bf16*>(out), scale, window, heads, kv_heads, page_size,
+            MllAttentionExtras{nullptr, 0, nullptr, 1.0f, 0});
+    }
     return check_launch("paged_attention_prefill");
 }
 
@@ -477,10 +524,25 @@ extern "C" int mll_paged_attention_prefill_tile() { return kPrefillTile; }
 
 
 
+extern "C" int mll_paged_attention_prefill_bias_rows() { return kPrefillBiasRows; }
+
 extern "C" int mll_paged_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                            const int32_t* block_table, int table_width, const int32_t* tiles,
                                            int n_tiles, const int32_t* positions, void* out, float scale, int window,
                                            int heads, int kv_heads, int head_dim, int page_size, hipStream_t stream) {
+    return mll_paged_attention_prefill_extra(q, k_cache, v_cache, block_table, table_width, tiles, n_tiles, positions, out, scale,
+                                             window, heads, kv_heads, head_dim, page_size, nullptr, stream);
+}
+
+extern "C" int mll_paged_attention_prefill_extra(const void* q, const void* k_cache, const void* v_cache,
+                                                 const int32_t* block_table, int table_width, const int32_t* tiles,
+                                                 int n_tiles, const int32_t* positions, void* out, float scale, int window,
+                                                 int heads, int kv_heads, int head_dim, int page_size,
+                                                 const MllAttentionExtras* extras, hipStream_t stream) {
+    MLL_REQUIRE(!extras || scale > 0.0f, "paged_attention_prefill: a bias or a sink needs a positive scale");
+    MLL_REQUIRE(!extras || !extras->bias || (extras->longest >= 0 && extras->longest < kPrefillBiasRows),
+                "paged_attention_prefill: the bias table has more rows than the kernel keeps");
+    MLL_REQUIRE(!extras || extras->out_stride >= static_cast<int64_t>(heads) * head_dim, "paged_attention_prefill: the output rows overlap");
     MLL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "paged_attention_prefill: heads must divide into kv_heads groups");
     MLL_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
                 "paged_attention_prefill: head_dim must be a multiple of 16 in [16, 256]");
@@ -490,7 +552,7 @@ extern "C" int mll_paged_attention_prefill(const void* q, const void* k_cache, c
 #define MLL_PREFILL_CASE(TILES)                                                                                      \
     case TILES:                                                                                                      \
         return launch_prefill<TILES>(q, k_cache, v_cache, block_table, table_width, tiles, n_tiles, positions, out,  \
-                                     scale, window, heads, kv_heads, page_size, stream);
+                                     scale, window, heads, kv_heads, page_size, extras, stream);
     switch (head_dim / 16) {
         MLL_PREFILL_CASE(1) MLL_PREFILL_CASE(2) MLL_PREFILL_CASE(3) MLL_PREFILL_CASE(4) MLL_PREFILL_CASE(5)
         MLL_PREFILL_CASE(6) MLL_PREFILL_CASE(7) MLL_PREFILL_CASE(8) MLL_PREFILL_CASE(9) MLL_PREFILL_CASE(10)

@@ -214,6 +214,31 @@ int mll_sample(const float* logits, const float* temperature, const int32_t* top
                hipStream_t stream);
 int64_t mll_sample_workspace(int n_rows, int vocab);
 
+// What the MFMA attention kernels take beyond scale and window (the *_extra entry points; null: nothing of it):
+// bias: float32 [longest + 1][heads], added to the scaled score of key j for a query at p as
+// bias[min(p - j, longest)][head] (null: none); sink: float32 [heads], exp(sink[head]) is one more term of the
+// softmax's denominator, without key or value (null: none); the result is multiplied by out_scale, and its rows
+// lie out_stride elements apart (at least heads * head_dim: it may be columns of a wider buffer).
+typedef struct MllAttentionExtras {
+    const float* bias;
+    int longest;
+    const float* sink;
+    float out_scale;
+    int64_t out_stride;
+} MllAttentionExtras;
+
+int mll_paged_attention_decode_extra(const void* q, const void* k_cache, const void* v_cache,
+                                     const int32_t* block_table, int table_width, const int32_t* seq_of_token,
+                                     const int32_t* positions, const int32_t* token_ids, void* out, float* part_o,
+                                     float* part_ml, float scale, int window, int n_tokens, int heads, int kv_heads,
+                                     int head_dim, int page_size, int n_splits, const MllAttentionExtras* extras,
+                                     hipStream_t stream);
+int mll_paged_attention_prefill_extra(const void* q, const void* k_cache, const void* v_cache,
+                                      const int32_t* block_table, int table_width, const int32_t* tiles,
+                                      int n_tiles, const int32_t* positions, void* out, float scale, int window,
+                                      int heads, int kv_heads, int head_dim, int page_size, const MllAttentionExtras* extras,
+                                      hipStream_t stream);
+
 // ---- several copies of the residual stream, a norm with a mean, a sinusoidal position vector ----------------
 
 // out[t, :] = table[ids[t], :] + wave(positions[t]) in float32, where entry 2i of the wave is
@@ -247,11 +272,12 @@ int mll_clamped_glu(const float* gate_up, void* out, int dtype, int n_tokens, in
 // (+ eps inside the root) and multiplied by q_weight / k_weight [key_dim] (both null: no norm); queries are then
 // multiplied by 1 + temp_coef * ln((p + 1) / temp_every + 1) (whole-number division) at position p
 // (temp_coef 0: not). Queries go to q_out [t][heads][key_dim]; keys and values into the pages
-// [slot][kv_head][dim] at slot_mapping[t] (negative: not stored).
+// [slot][kv_head][dim] at slot_mapping[t] (negative: not stored), or, with tiled_page_size > 0 (the positions of a
+// page; key_dim == value_dim), into pages in the MFMA kernels' order (cache_layout.h).
 int mll_qk_norm_store(const float* qkv, int n_parts, int64_t part_stride, const float* q_weight, const float* k_weight,
                       float eps, const int32_t* positions, const int32_t* slot_mapping, float temp_coef, int temp_every,
                       void* q_out, void* k_pages, void* v_pages, int dtype, int n_tokens, int heads, int kv_heads, int key_dim,
-                      int value_dim, hipStream_t stream);
+                      int value_dim, int tiled_page_size, hipStream_t stream);
 
 // Causal attention of every token over its request's pages: score_j = (q . k_j) * scale + bias[min(p - j, longest)][head]
 // (bias null: none; float32 [longest + 1][heads]); softmax over j <= p with exp(sink[head]) added to the denominator

@@ -600,6 +600,44 @@ def gemm_bf16_split(x: torch.Tensor, weight: torch.Tensor, parts: int) -> torch.
     return torch.bmm(a, b, out_dtype=torch.float32)
 
 
+class _AttentionExtras(ctypes.Structure):
+    _fields_ = [("bias", ctypes.c_void_p), ("longest", ctypes.c_int), ("sink", ctypes.c_void_p),
+                ("out_scale", ctypes.c_float), ("out_stride", ctypes.c_int64)]
+
+
+class AttentionExtras(NamedTuple):
+    """What the MFMA attention kernels take beyond scale and window: ``bias`` float32 ``[distances, heads]`` added to
+    the scaled scores by ``min(distance, last row)``; ``sink`` float32 ``[heads]``, one more term ``exp(sink)`` of the
+    softmax's denominator; a factor on the result."""
+    bias: Optional[torch.Tensor] = None
+    sink: Optional[torch.Tensor] = None
+    out_scale: float = 1.0
+
+
+def prefill_bias_rows() -> int:
+    """The most rows of a bias table that the prefill kernel takes."""
+    return int(library.load().mll_paged_attention_prefill_bias_rows())
+
+
+def _extras_argument(extras: Optional[AttentionExtras], heads: int, head_dim: int, out: torch.Tensor):
+    if extras is None:
+        _need(out.is_contiguous(), "the attention output must be contiguous")
+        return None
+    longest = 0
+    if extras.bias is not None:
+        _device_tensor(extras.bias, "bias by distance", torch.float32)
+        _need(extras.bias.dim() == 2 and extras.bias.shape[1] == heads and extras.bias.shape[0] >= 1, "the bias is [distances, heads]")
+        longest = extras.bias.shape[0] - 1
+    if extras.sink is not None:
+        _device_tensor(extras.sink, "sink", torch.float32)
+        _need(tuple(extras.sink.shape) == (heads,), "one sink a head")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == heads * head_dim, "the output is [tokens, heads * head_dim] with unit column stride")
+    stride = max(out.stride(0), heads * head_dim)
+    return ctypes.byref(_AttentionExtras(extras.bias.data_ptr() if extras.bias is not None else None, longest,
+                                         extras.sink.data_ptr() if extras.sink is not None else None,
+                                         float(extras.out_scale), stride))
+
+
 def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
     """How many splits of the keys: about one workgroup per compute unit, at least 512 keys each, and 1024 where
     that alone fills the GPU (measured on MI355X: a wave keeps two pairs of key tiles on their way, so few long
@@ -614,7 +652,8 @@ def decode_splits(n_tokens: int, kv_heads: int, longest: int) -> int:
 def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                            seq_of_token: torch.Tensor, positions: torch.Tensor, scale: float, window: int,
                            heads: int, kv_heads: int, head_dim: int, n_splits: int,
-                           out: Optional[torch.Tensor] = None, token_ids: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           out: Optional[torch.Tensor] = None, token_ids: Optional[torch.Tensor] = None,
+                           extras: Optional[AttentionExtras] = None) -> torch.Tensor:
     """The MFMA kernel for bfloat16 queries that each attend alone (one token per request).
 
     ``token_ids`` restricts the work to those rows of ``q`` (the other rows of ``out`` are left alone)."""
@@ -635,16 +674,16 @@ def paged_attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         n_tokens = token_ids.shape[0]
     if out is None:
         out = torch.empty_like(q)
-    _device_tensor(out, "attention output", q.dtype)
-    _need(out.shape == q.shape, "attention output must have the queries' shape")
+    _need(out.is_cuda and out.dtype == q.dtype and out.shape == q.shape, "attention output must have the queries' shape and dtype")
+    extra = _extras_argument(extras, heads, head_dim, out)
     part_o = part_ml = None
     if n_splits > 1:
         part_o = torch.empty((n_tokens, heads, n_splits, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((n_tokens, heads, n_splits, 2), dtype=torch.float32, device=q.device)
-    _check(lib.mll_paged_attention_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
-                                          _ptr(seq_of_token), _ptr(positions), _ptr(token_ids), _ptr(out), _ptr(part_o),
-                                          _ptr(part_ml), ctypes.c_float(scale), int(window), n_tokens, heads, kv_heads,
-                                          head_dim, page_size, n_splits, _stream()), lib)
+    _check(lib.mll_paged_attention_decode_extra(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                                                _ptr(seq_of_token), _ptr(positions), _ptr(token_ids), ctypes.c_void_p(out.data_ptr()),
+                                                _ptr(part_o), _ptr(part_ml), ctypes.c_float(scale), int(window), n_tokens, heads,
+                                                kv_heads, head_dim, page_size, n_splits, extra, _stream()), lib)
     return out
 
 
@@ -680,7 +719,8 @@ def pair_query_tiles(tiles: Sequence[Tuple[int, int, int, int]], adjacent: bool 
 
 def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                             query_tiles: torch.Tensor, positions: torch.Tensor, scale: float, window: int,
-                            heads: int, kv_heads: int, head_dim: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            heads: int, kv_heads: int, head_dim: int, out: Optional[torch.Tensor] = None,
+                            extras: Optional[AttentionExtras] = None) -> torch.Tensor:
     """The MFMA kernel for bfloat16 portions of prompts; ``query_tiles`` rows are (request, first token, tokens,
     first token, tokens): two tiles of up to ``QUERY_TILE`` tokens of the request (``pair_query_tiles``)."""
     lib = library.load()
@@ -693,17 +733,19 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     _need(positions.shape[0] == q.shape[0], "positions must hold one entry per token")
     if out is None:
         out = torch.empty_like(q)
-    _device_tensor(out, "attention output", q.dtype)
-    _need(out.shape == q.shape, "attention output must have the queries' shape")
-    _check(lib.mll_paged_attention_prefill(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
-                                           _ptr(query_tiles), query_tiles.shape[0], _ptr(positions), _ptr(out),
-                                           ctypes.c_float(scale), int(window), heads, kv_heads, head_dim, page_size,
-                                           _stream()), lib)
+    _need(out.is_cuda and out.dtype == q.dtype and out.shape == q.shape, "attention output must have the queries' shape and dtype")
+    extra = _extras_argument(extras, heads, head_dim, out)
+    _need(extras is None or extras.bias is None or extras.bias.shape[0] <= prefill_bias_rows(), "the bias table has too many rows for the prefill kernel")
+    _check(lib.mll_paged_attention_prefill_extra(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
+                                                 _ptr(query_tiles), query_tiles.shape[0], _ptr(positions), ctypes.c_void_p(out.data_ptr()),
+                                                 ctypes.c_float(scale), int(window), heads, kv_heads, head_dim, page_size,
+                                                 extra, _stream()), lib)
     return out
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, view, ctx,
-                    scale: float, window: int, heads: int, kv_heads: int, head_dim: int, planner=None) -> torch.Tensor:
+                    scale: float, window: int, heads: int, kv_heads: int, head_dim: int, planner=None,
+                    extras: Optional[AttentionExtras] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the step's queries over their requests' pages; chooses the kernel for the batch's shape.
 
     bfloat16 with a head size in steps of 16: the MFMA kernels, split over the keys when every request brings
@@ -711,26 +753,29 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     holds the tiles). Everything else (float32, other head sizes): the plain kernel.
     """
     mfma_fits = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
+    _need(mfma_fits or (extras is None and out is None), "a bias, a sink or an output of its own need the MFMA kernels")
     if mfma_fits and ctx.max_count == 1:
         longest = max(ctx.planned_total, ctx.max_total)
         visible = min(longest, window) if window > 0 else longest
         splits = decode_splits(ctx.n_tokens, kv_heads, visible)
         return paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
-                                      scale, window, heads, kv_heads, head_dim, splits)
+                                      scale, window, heads, kv_heads, head_dim, splits, out=out, extras=extras)
     if mfma_fits:
         # Portions go to the tiled kernel; requests that bring one token, if any, to the split kernel.
         _need(planner is not None, "portions of prompts need the attention part's planner for their tiles")
         plan = ctx.plan_of(planner)
-        out = torch.empty_like(q)
+        if out is None:
+            out = torch.empty_like(q)
         if plan.tiles.shape[0] > 0:
             paged_attention_prefill(q, k_cache, v_cache, view.block_table, plan.tiles, ctx.positions,
-                                    scale, window, heads, kv_heads, head_dim, out=out)
+                                    scale, window, heads, kv_heads, head_dim, out=out, extras=extras)
         if plan.single_tokens.shape[0] > 0:
             longest = max(plan.max_single_total, ctx.planned_total) if ctx.fixed else plan.max_single_total
             visible = min(longest, window) if window > 0 else longest
             splits = decode_splits(plan.single_tokens.shape[0], kv_heads, visible)
             paged_attention_decode(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
-                                   scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens)
+                                   scale, window, heads, kv_heads, head_dim, splits, out=out, token_ids=plan.single_tokens,
+                                   extras=extras)
         return out
     return paged_attention_rowwise(q, k_cache, v_cache, view.block_table, ctx.seq_of_token, ctx.positions,
                                    scale, window, heads, kv_heads, head_dim, longest=max(ctx.planned_total, ctx.max_total),
@@ -1008,6 +1053,7 @@ def stream_copies(h: torch.Tensor, copies: int) -> torch.Tensor:
 
 
 MAX_STREAMS = 8
+MFMA_BIAS_ROWS = 4096     # rows of a bias table that the MFMA prefill kernel keeps in LDS (csrc/attention_prefill.hip)
 
 
 def stream_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype, rms: bool = False,
@@ -1087,9 +1133,10 @@ def _parts_of(tensor: torch.Tensor, name: str) -> Tuple[int, int]:
 def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                   positions: torch.Tensor, slot_mapping: torch.Tensor, temp_coef: float, temp_every: int,
                   k_pages: torch.Tensor, v_pages: torch.Tensor, heads: int, kv_heads: int, key_dim: int, value_dim: int,
-                  out_dtype: torch.dtype) -> torch.Tensor:
+                  out_dtype: torch.dtype, tiled_page_size: int = 0) -> torch.Tensor:
     """Norm of queries and keys over their head, the queries' factor by position, keys and values into their pages
-    (``[page, position, kv_head, dim]``); returns the queries ``[tokens, heads * key_dim]``."""
+    (``[page, position, kv_head, dim]``, or with ``tiled_page_size`` the pages of ``cache.layout`` with that many
+    positions each); returns the queries ``[tokens, heads * key_dim]``."""
     lib = library.load()
     n_parts, part_stride = _parts_of(qkv, "q/k/v")
     n_tokens = qkv.shape[-2]
@@ -1103,14 +1150,18 @@ def qk_norm_store(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight:
             _need(tuple(weight.shape) == (key_dim,), f"{name} must have the head's size")
     _device_tensor(k_pages, "key pages", out_dtype)
     _device_tensor(v_pages, "value pages", out_dtype)
-    _need(k_pages.dim() == 4 and tuple(k_pages.shape[2:]) == (kv_heads, key_dim), "key pages are [page, position, kv_head, key_dim]")
-    _need(v_pages.dim() == 4 and tuple(v_pages.shape[2:]) == (kv_heads, value_dim) and v_pages.shape[:2] == k_pages.shape[:2],
-          "value pages are [page, position, kv_head, value_dim]")
+    if tiled_page_size:
+        _need(key_dim == value_dim, "tiled pages hold keys and values of one width")
+        _check_pages(k_pages, v_pages, out_dtype, kv_heads, key_dim, tiled_page_size)
+    else:
+        _need(k_pages.dim() == 4 and tuple(k_pages.shape[2:]) == (kv_heads, key_dim), "key pages are [page, position, kv_head, key_dim]")
+        _need(v_pages.dim() == 4 and tuple(v_pages.shape[2:]) == (kv_heads, value_dim) and v_pages.shape[:2] == k_pages.shape[:2],
+              "value pages are [page, position, kv_head, value_dim]")
     q_out = torch.empty((n_tokens, heads * key_dim), dtype=out_dtype, device=qkv.device)
     _check(lib.mll_qk_norm_store(_ptr(qkv), n_parts, ctypes.c_int64(part_stride), _ptr(q_weight), _ptr(k_weight),
                                  ctypes.c_float(eps), _ptr(positions), _ptr(slot_mapping), ctypes.c_float(temp_coef),
                                  int(temp_every), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _code(out_dtype), n_tokens,
-                                 heads, kv_heads, key_dim, value_dim, _stream()), lib)
+                                 heads, kv_heads, key_dim, value_dim, int(tiled_page_size), _stream()), lib)
     return q_out
 
 

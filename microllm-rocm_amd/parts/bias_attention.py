@@ -10,7 +10,12 @@ longest distance ``D``: ``bucket(n) = n`` below ``B / 2``, else ``min(B - 1, B/2
 * (B - B/2)))``. The softmax's denominator also holds ``exp(sink[h])``, which has no key and no value.
 
 Every distance from ``D`` on falls into the last bucket, so the table is unrolled once, at load, into one row per
-distance up to ``D`` and the kernel indexes it with ``min(i - j, D)``.
+distance up to ``D`` and the kernels index it with ``min(i - j, D)``.
+
+In bfloat16, with keys and values of one width that is a multiple of 16, the pages are the paged attention's own
+(``PagedKVNeed``) and the attention runs on its MFMA kernels, which take the bias, the sink and the result's factor
+as extras; everything else (float32, two widths, other sizes) lies in plain pages (``PagedKeyValueNeed``) and runs on
+the kernel that takes a wave per token and head.
 """
 from __future__ import annotations
 
@@ -20,7 +25,8 @@ from typing import Dict, Mapping, Optional
 import torch
 
 from ..ops import kernels
-from .base import MATRIX, Mixer, PagedKeyValueNeed, Runtime, TensorDecl, VECTOR
+from .attention import QueryTilePlanner
+from .base import MATRIX, Mixer, PagedKeyValueNeed, PagedKVNeed, Runtime, TensorDecl, VECTOR
 from .linear import Weight, linear
 from .registry import register_part
 from .spec import PartSpec
@@ -58,6 +64,10 @@ class BucketBiasAttention(Mixer):
             raise ValueError("heads must divide into kv_heads groups")
         if self.bias_rows and self.bias_max <= self.bias_rows // 2:
             raise ValueError("bias_max must lie beyond the distances that have a bucket of their own")
+        # the paged attention's pages and MFMA kernels, where they fit (the bias column must fit the prefill kernel's LDS)
+        self.tiled = (runtime.dtype == torch.bfloat16 and self.key_dim == self.value_dim and self.key_dim % 16 == 0
+                      and self.key_dim <= 256 and self.bias_max + 1 <= kernels.MFMA_BIAS_ROWS)
+        self.planner = QueryTilePlanner(False) if self.tiled else None
         self.qkv_weight: Optional[Weight] = None
         self.o_tensor: Optional[torch.Tensor] = None
         self.o_weight: Optional[Weight] = None
@@ -103,13 +113,20 @@ class BucketBiasAttention(Mixer):
         tensor, self.o_tensor = self.o_tensor, None
         return tensor
 
+    def step_planner(self):
+        return self.planner
+
     def cache_need(self):
+        if self.tiled:
+            return PagedKVNeed(self.kv_heads, self.key_dim)
         return PagedKeyValueNeed(self.kv_heads, self.key_dim, self.value_dim)
 
     def flops(self, tokens: int) -> float:
         pairs = tokens * (tokens + 1) / 2
-        own = 2.0 * tokens * self.hidden * ((self.heads + self.kv_heads) * self.key_dim + (self.kv_heads + self.heads) * self.value_dim)
-        return own + 2.0 * self.heads * (self.key_dim + self.value_dim) * pairs
+        columns = (self.heads + self.kv_heads) * self.key_dim + self.kv_heads * self.value_dim
+        if self.o_tensor is not None or self.o_weight is not None:      # else the mixer that took the projection counts it
+            columns += self.heads * self.value_dim
+        return 2.0 * tokens * self.hidden * columns + 2.0 * self.heads * (self.key_dim + self.value_dim) * pairs
 
     def forward_inner(self, x, ctx, cache, out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
         """The heads' results side by side, ``[tokens, heads * value_dim]`` times ``out_scale``, before the output
@@ -118,7 +135,13 @@ class BucketBiasAttention(Mixer):
         qkv = linear(x, self.qkv_weight, out_dtype=torch.float32, partials=True)     # rounded once, after norm and factor
         q = kernels.qk_norm_store(qkv, self.q_norm, self.k_norm, self.eps, ctx.positions, view.slot_mapping, self.temp_coef,
                                   self.temp_every, cache.k, cache.v, self.heads, self.kv_heads, self.key_dim, self.value_dim,
-                                  self.runtime.dtype)
+                                  self.runtime.dtype, tiled_page_size=view.page_size if self.tiled else 0)
+        if self.tiled:
+            if out is None:
+                out = torch.empty((x.shape[0], self.heads * self.value_dim), dtype=self.runtime.dtype, device=x.device)
+            extras = kernels.AttentionExtras(self.bias, self.sink, out_scale)
+            return kernels.paged_attention(q, cache.k, cache.v, view, ctx, self.scale, 0, self.heads, self.kv_heads, self.key_dim,
+                                           planner=self.planner, extras=extras, out=out)
         return kernels.bias_attention(q, cache.k, cache.v, view.block_table, ctx.seq_of_token, ctx.positions, self.bias,
                                       self.sink, self.scale, out_scale, self.heads, self.kv_heads, self.key_dim,
                                       self.value_dim, out=out)

@@ -82,7 +82,8 @@ class GatedLinearAttention(Mixer):
 
     def flops(self, tokens: int) -> float:
         keys, values = self.heads * self.key_dim, self.heads * self.value_dim
-        products = 2.0 * tokens * (self.hidden * (2 * keys + 3 * values + self.rank) + keys * self.rank)
+        outputs = values if self.o_tensor is not None or self.o_weight is not None else 0
+        products = 2.0 * tokens * (self.hidden * (2 * keys + 2 * values + outputs + self.rank) + keys * self.rank)
         return products + 5.0 * tokens * self.heads * self.key_dim * self.value_dim
 
     def forward_inner(self, x, ctx, cache, out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:

@@ -46,8 +46,19 @@ TINY_C = SiditarConfig(
                LinearAttentionConfig(heads=1, dim=16, vdim=32, tau=6.0, decay_rank=6), (0.8, 1.2), DenseMlpConfig(72, 3.0)),
     ))
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-SEEDS = {"A": 11, "B": 12, "C": 13}
+# Keys and values of one width that is a multiple of 16: in bfloat16 these layers take the paged attention's own pages
+# and MFMA kernels; two streams; grouped kv heads; a bias table whose longest distance is shorter than the tests' prompts.
+TINY_D = SiditarConfig(
+    vocab=150, width=64, norm_eps=1e-6, streams=2, loop=LoopConfig(0, 1, 2),
+    layers=(
+        _layer(BiasAttentionConfig(heads=4, kv_heads=2, dim=32, vdim=32, scale=0.2, bias_max=70, temp_coef=0.5, temp_every=8, bias_rows=12),
+               LinearAttentionConfig(heads=2, dim=16, vdim=32, tau=8.0, decay_rank=4), (0.8, 1.1), DenseMlpConfig(96, 1.5)),
+        _layer(BiasAttentionConfig(heads=2, kv_heads=2, dim=16, vdim=16, scale=0.3, bias_max=20, temp_coef=0.3, temp_every=3, bias_rows=8),
+               LinearAttentionConfig(heads=3, dim=8, vdim=16, tau=2.0, decay_rank=2), (1.2, 0.9), DenseMlpConfig(64, 2.0)),
+    ))
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+SEEDS = {"A": 11, "B": 12, "C": 13, "D": 14}
 STDS = {"std": 0.08, "norm_std": 0.1, "connection_std": 0.15, "bias_std": 0.7}
 
 

@@ -234,6 +234,95 @@ def test_query_and_key_norm_and_factor_by_position():
     assert np.abs(got - want).max() < 2e-5
 
 
+def attention_through_mfma(q, k, v, scale, table, longest, sink, portions_of, page_size=16, splits=None, out_scale=1.0):
+    """The same through the paged attention's pages and MFMA kernels (bfloat16, one width for keys and values):
+    portions of several tokens go to the tiled kernel, single tokens to the kernel that splits the keys."""
+    from microllm_rocm_amd.cache.layout import key_page_shape, value_page_shape
+    from microllm_rocm_amd.ops import kernels
+    n, heads, dim = q.shape
+    kv_heads = k.shape[1]
+    blocks = -(-n // page_size)
+    pages = [2 + 3 * block for block in reversed(range(blocks))]
+    k_pages = torch.zeros(key_page_shape(3 * blocks + 2, kv_heads, page_size, dim), dtype=torch.bfloat16, device="cuda")
+    v_pages = torch.zeros(value_page_shape(3 * blocks + 2, kv_heads, page_size, dim), dtype=torch.bfloat16, device="cuda")
+    bias = None
+    if table is not None:
+        bias = device(np.stack([table[plain.bucket_of(distance, table.shape[0], longest)] for distance in range(longest + 1)]))
+    block_table = device([pages], torch.int32)
+    extras = kernels.AttentionExtras(bias, device(sink) if sink is not None else None, out_scale)
+    outputs, position = [], 0
+    for count in portions_of:
+        count = min(count, n - position)
+        if count <= 0:
+            break
+        rows = slice(position, position + count)
+        qkv = np.concatenate([q[rows].reshape(count, -1), k[rows].reshape(count, -1), v[rows].reshape(count, -1)], axis=1)
+        positions = device(np.arange(position, position + count), torch.int32)
+        slots = device([pages[p // page_size] * page_size + p % page_size for p in range(position, position + count)], torch.int32)
+        queries = kernels.qk_norm_store(device(qkv), None, None, 1e-6, positions, slots, 0.0, 1, k_pages, v_pages, heads, kv_heads,
+                                        dim, dim, torch.bfloat16, tiled_page_size=page_size)
+        wide = torch.zeros((count, heads * dim + 8), dtype=torch.bfloat16, device="cuda")     # the result as columns of a wider buffer
+        out = wide[:, 8:]
+        requests = device(np.zeros(count), torch.int32)
+        if count == 1:
+            kernels.paged_attention_decode(queries, k_pages, v_pages, block_table, requests, positions, scale, 0, heads, kv_heads, dim,
+                                           splits or kernels.decode_splits(1, kv_heads, position + 1), out=out, extras=extras)
+        else:
+            tiles = [(0, offset, min(kernels.QUERY_TILE, count - offset), position + offset) for offset in range(0, count, kernels.QUERY_TILE)]
+            plan = device(np.asarray(kernels.pair_query_tiles(tiles)).reshape(-1, 5), torch.int32)
+            kernels.paged_attention_prefill(queries, k_pages, v_pages, block_table, plan, positions, scale, 0, heads, kv_heads, dim,
+                                            out=out, extras=extras)
+        assert float(wide[:, :8].abs().max()) == 0.0
+        outputs.append(out.float().cpu().numpy().reshape(count, heads, dim))
+        position += count
+    return np.concatenate(outputs)
+
+
+def as_bf16(array):
+    return torch.as_tensor(array, dtype=torch.float32).to(torch.bfloat16).to(torch.float64).numpy()
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,n", [(4, 2, 32, 300), (2, 2, 16, 77), (6, 1, 48, 150), (1, 1, 128, 270)])
+def test_mfma_attention_with_bias_and_sink(heads, kv_heads, dim, n):
+    rng = np.random.default_rng(dim + n)
+    q, k, v = (as_bf16(rng.normal(size=shape)) for shape in ((n, heads, dim), (n, kv_heads, dim), (n, kv_heads, dim)))
+    table, sink = rng.normal(size=(10, heads)) * 2, rng.normal(size=heads)
+    want = plain.bias_sink_attention(q, k, v, 0.2, table, 27, sink) * 1.5
+    for portions_of in ([n], [140, 3] + [1] * 20 + [200], [1] * 40 + [2, 129, 1, 1, 1, 500]):
+        got = attention_through_mfma(q, k, v, 0.2, table, 27, sink, portions_of, out_scale=1.5)
+        assert np.abs(got - want).max() < 0.03 * np.abs(want).max(), portions_of       # weights and results are bfloat16
+    got = attention_through_mfma(q, k, v, 0.2, table, 27, sink, [n - 1, 1], splits=3, out_scale=1.5)
+    assert np.abs(got - want).max() < 0.03 * np.abs(want).max()
+    want = plain.bias_sink_attention(q, k, v, 0.2, None, 0, None)
+    assert np.abs(attention_through_mfma(q, k, v, 0.2, None, 0, None, [n]) - want).max() < 0.03 * np.abs(want).max()
+
+
+def test_mfma_bias_buckets_sink_and_far_keys():
+    """The constructed cases of the plain kernel's tests through the MFMA kernels: weights from the bias alone at
+    every distance up to beyond the longest, a sink that takes weight, one far key that decides."""
+    rows, longest, n = 8, 21, 200
+    table = (np.arange(rows)[:, None] * 0.9) * np.array([[1.0, -1.0]])
+    q, k = np.zeros((n, 2, 16)), np.zeros((n, 1, 16))
+    v = as_bf16(np.random.default_rng(0).normal(size=(n, 1, 16)))
+    sink = np.array([0.5, -0.5])
+    want = plain.bias_sink_attention(q, k, v, 1.0, table, longest, sink)
+    for portions_of in ([n], [150] + [1] * 50, [1] * 30 + [170]):
+        got = attention_through_mfma(q, k, v, 1.0, table, longest, sink, portions_of)
+        assert np.abs(got - want).max() < 0.02, portions_of
+    v = np.ones((n, 1, 16))
+    got = attention_through_mfma(q, k, v, 1.0, None, 0, np.array([math.log(3.0), 30.0]), [100] + [1] * 100)
+    assert np.abs(got[:, 0, 0] - np.array([(i + 1) / (i + 4) for i in range(n)])).max() < 0.01 and np.abs(got[:, 1]).max() < 1e-9
+    for far in (0, 1, 31, 32, 127, 128, 150):
+        rng = np.random.default_rng(far)
+        q, k, v = as_bf16(rng.normal(size=(n, 1, 16)) * 0.1), as_bf16(rng.normal(size=(n, 1, 16)) * 0.1), as_bf16(rng.normal(size=(n, 1, 16)))
+        q[-1, 0] = 0.0
+        q[-1, 0, 3] = 6.0
+        k[far, 0, 3] = 6.0
+        for portions_of in ([n], [n - 1, 1]):
+            got = attention_through_mfma(q, k, v, 1.0, None, 0, np.zeros(1), portions_of)
+            assert np.abs(got[-1, 0] - v[far, 0]).max() < 0.02, (far, portions_of)
+
+
 @pytest.mark.parametrize("heads,dim,vdim,rank,tau", [(3, 16, 8, 5, 4.0), (1, 40, 24, 3, 1.5), (2, 8, 72, 1, 16.0), (1, 130, 5, 2, 1.0)])
 def test_linear_attention_walk(heads, dim, vdim, rank, tau):
     """Decays, the walk with carried state and the gate: two requests in one step, then both continued one token at
@@ -292,7 +381,7 @@ def test_linear_attention_walk(heads, dim, vdim, rank, tau):
 
 # ---- the engine ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_whole_decode_and_portions(tmp_path_factory, tmp_path, which, dtype):
     folder, config, weights = model_for(tmp_path_factory, which)
     requests = {"long": tokens_for(1, 150, config["vocab"]), "short": tokens_for(2, 37, config["vocab"]), "one": tokens_for(3, 1, config["vocab"])}
@@ -309,7 +398,7 @@ def test_whole_decode_and_portions(tmp_path_factory, tmp_path, which, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "C"])
+@pytest.mark.parametrize("which", ["A", "C", "D"])
 def test_mixed_batches_on_reused_pages_and_slots(tmp_path_factory, tmp_path, which, dtype):
     folder, config, weights = model_for(tmp_path_factory, which)
     lengths = [90, 41, 130, 2, 67, 25, 110, 58]
@@ -366,7 +455,7 @@ def test_long_decoding_through_graphs(tmp_path_factory, which):
         assert row_errors(np.stack(rows[name]), want).max() < F32_BOUND
 
 
-@pytest.mark.parametrize("which", ["A", "C"])
+@pytest.mark.parametrize("which", ["A", "C", "D"])
 def test_greedy_generation_through_the_scheduler(tmp_path_factory, which):
     from microllm_rocm_amd import Engine, GenerationConfig, generate, generate_serial
     folder, config, weights = model_for(tmp_path_factory, which)
