@@ -32,7 +32,9 @@ __global__ void gla_decay_kernel(const float* __restrict__ proj, int64_t proj_st
 }
 
 // One wave a (request, head, group of value channels). lane = column_in_group * lanes_a_column + r; lane r of a
-// column keeps key channels r, r + lanes_a_column, ... (kStateRowsALane of them).
+// column keeps the key channels 8 r .. 8 r + 7. A token's result is the sum over a lane's channels in order, then
+// over the column's lanes by exchanges 1, 2, 4, .. apart: both kernels below add in this order, so a request gives
+// the same bits whichever of them walks its tokens.
 __global__ void __launch_bounds__(kWave)
 gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                 const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
@@ -52,7 +54,7 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
     float s[kStateRowsALane];
 #pragma unroll
     for (int m = 0; m < kStateRowsALane; ++m) {
-        const int i = r + m * lanes_a_column;
+        const int i = 8 * r + m;
         s[m] = i < key_dim ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
     }
     const int channels = heads * key_dim;
@@ -62,7 +64,7 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
         const float* decays = decay + static_cast<int64_t>(token) * channels + head * key_dim;
 #pragma unroll
         for (int m = 0; m < kStateRowsALane; ++m) {
-            const int i = r + m * lanes_a_column;
+            const int i = 8 * r + m;
             const bool in = i < key_dim;
             a_next[m] = in ? decays[i] : 0.0f;
             k_next[m] = in ? row[k_offset + head * key_dim + i] : 0.0f;
@@ -89,7 +91,119 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
     if (!live) return;
 #pragma unroll
     for (int m = 0; m < kStateRowsALane; ++m) {
-        const int i = r + m * lanes_a_column;
+        const int i = 8 * r + m;
+        if (i < key_dim) mine[static_cast<int64_t>(i) * value_dim] = s[m];
+    }
+}
+
+// The same walk for portions of many tokens: a wave brings tiles of tokens (decays, keys, queries of its head, the
+// values of its columns) from memory straight into LDS, the next tile on its way while it walks this one, and reads
+// its eight key channels of a token as two 16-byte pieces. The walk over a request's tokens stays in order, with the
+// same operations per token in the same order as above; only where the operands come from differs.
+constexpr int kScanTileFloats = 1024;                    // of each of decays, keys, queries (and at most of values) in a tile
+constexpr int kScanCalls = kScanTileFloats / kWave;      // loads of 4 bytes a lane that bring one of them
+constexpr int kScanBufferFloats = 4 * kScanTileFloats;
+
+__global__ void __launch_bounds__(kWave)
+gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
+                      const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
+                      const int32_t* __restrict__ slots, float* __restrict__ out, int heads, int key_dim, int value_dim,
+                      int lanes_a_column, int tile_tokens, float q_scale) {
+    __shared__ __align__(16) float buffer_even[kScanBufferFloats];
+    __shared__ __align__(16) float buffer_odd[kScanBufferFloats];
+    const int seq = blockIdx.x;
+    const int head = blockIdx.y;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    if (last <= first) return;
+    const int lane = threadIdx.x;
+    const int r = lane % lanes_a_column;
+    const int columns = kWave / lanes_a_column;              // of this wave
+    const int column_in_group = lane / lanes_a_column;
+    const int column = blockIdx.z * columns + column_in_group;
+    const bool live = column < value_dim;
+    const int safe_column = live ? column : 0;
+    const int row_floats = (key_dim + 7) / 8 * 8;            // a token's row of key channels in LDS
+    const int slot = slots[seq];
+    float* mine = state + ((static_cast<int64_t>(slot) * heads + head) * key_dim) * value_dim + safe_column;
+    float s[kStateRowsALane];
+    bool valid[kStateRowsALane];
+#pragma unroll
+    for (int m = 0; m < kStateRowsALane; ++m) {
+        const int i = 8 * r + m;
+        valid[m] = i < key_dim;
+        s[m] = valid[m] ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
+    }
+    // Nothing that is read from LDS may be a stray bit pattern: places that no load fills are read beside others.
+    for (int index = lane; index < kScanBufferFloats; index += kWave) buffer_even[index] = buffer_odd[index] = 0.0f;
+    __syncthreads();
+    // Which token of a tile and which channel each of this lane's loads brings (the same for every tile).
+    int token_of[kScanCalls], channel_of[kScanCalls];
+#pragma unroll
+    for (int j = 0; j < kScanCalls; ++j) {
+        const int element = j * kWave + lane;
+        token_of[j] = element / row_floats;
+        channel_of[j] = min(element % row_floats, key_dim - 1);
+    }
+    const int channels = heads * key_dim;
+    const int value_calls = (tile_tokens * columns + kWave - 1) / kWave;
+    auto fetch = [&](int tile_first, float* buffer) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < kScanCalls; ++j) {
+            if (j * kWave >= tile_tokens * row_floats) break;
+            const int64_t token = min(tile_first + token_of[j], last - 1);
+            const float* row = proj + token * proj_stride + head * key_dim + channel_of[j];
+            __builtin_amdgcn_global_load_lds(decay + token * channels + head * key_dim + channel_of[j], buffer + j * kWave, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(row + k_offset, buffer + kScanTileFloats + j * kWave, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds(row + q_offset, buffer + 2 * kScanTileFloats + j * kWave, 4, 0, 0);
+        }
+        for (int j = 0; j < value_calls; ++j) {
+            const int element = j * kWave + lane;
+            const int64_t token = min(tile_first + element / columns, last - 1);
+            const int wanted = min(static_cast<int>(blockIdx.z) * columns + element % columns, value_dim - 1);
+            __builtin_amdgcn_global_load_lds(proj + token * proj_stride + v_offset + head * value_dim + wanted,
+                                             buffer + 3 * kScanTileFloats + j * kWave, 4, 0, 0);
+        }
+    };
+    auto walk = [&](int tile_first, const float* buffer) __attribute__((always_inline)) {
+        const int count = min(tile_tokens, last - tile_first);
+        for (int t = 0; t < count; ++t) {
+            const float* row = buffer + t * row_floats + 8 * r;
+            float a[8], k[8], q[8];
+            *reinterpret_cast<float4*>(a) = *reinterpret_cast<const float4*>(row);
+            *reinterpret_cast<float4*>(a + 4) = *reinterpret_cast<const float4*>(row + 4);
+            *reinterpret_cast<float4*>(k) = *reinterpret_cast<const float4*>(row + kScanTileFloats);
+            *reinterpret_cast<float4*>(k + 4) = *reinterpret_cast<const float4*>(row + kScanTileFloats + 4);
+            *reinterpret_cast<float4*>(q) = *reinterpret_cast<const float4*>(row + 2 * kScanTileFloats);
+            *reinterpret_cast<float4*>(q + 4) = *reinterpret_cast<const float4*>(row + 2 * kScanTileFloats + 4);
+            const float v = buffer[3 * kScanTileFloats + t * columns + column_in_group];
+            float partial = 0.0f;
+#pragma unroll
+            for (int m = 0; m < kStateRowsALane; ++m) {
+                s[m] = fmaf(a[m], s[m], (valid[m] ? k[m] : 0.0f) * v);
+                partial = fmaf(s[m], q[m] * q_scale, partial);
+            }
+            for (int offset = 1; offset < lanes_a_column; offset <<= 1) partial += __shfl_xor(partial, offset, kWave);
+            if (live && r == 0) out[(static_cast<int64_t>(tile_first + t) * heads + head) * value_dim + column] = partial;
+        }
+    };
+    fetch(first, buffer_even);
+    for (int tile_first = first; tile_first < last;) {
+        wait_for_loads();
+        __syncthreads();
+        if (tile_first + tile_tokens < last) fetch(tile_first + tile_tokens, buffer_odd);
+        walk(tile_first, buffer_even);
+        tile_first += tile_tokens;
+        if (tile_first >= last) break;
+        wait_for_loads();
+        __syncthreads();
+        if (tile_first + tile_tokens < last) fetch(tile_first + tile_tokens, buffer_even);
+        walk(tile_first, buffer_odd);
+        tile_first += tile_tokens;
+    }
+    if (!live) return;
+#pragma unroll
+    for (int m = 0; m < kStateRowsALane; ++m) {
+        const int i = 8 * r + m;
         if (i < key_dim) mine[static_cast<int64_t>(i) * value_dim] = s[m];
     }
 }
@@ -143,7 +257,7 @@ int mll_gla_decay(const float* proj, int64_t proj_stride, int low_offset, int ra
 
 int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset, const float* decay,
                  float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
-                 int value_dim, float q_scale, hipStream_t stream) {
+                 int value_dim, float q_scale, int long_portions, hipStream_t stream) {
     MLL_REQUIRE(n_seqs >= 0 && heads > 0 && key_dim > 0 && value_dim > 0, "gla_scan: sizes must be positive");
     MLL_REQUIRE(key_dim <= kStateRowsALane * kWave, "gla_scan: key heads wider than 512 are not supported");
     MLL_REQUIRE(q_offset >= 0 && k_offset >= 0 && v_offset >= 0 && q_offset + heads * key_dim <= proj_stride &&
@@ -155,6 +269,15 @@ int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_off
     const int columns_a_wave = kWave / lanes_a_column;
     MLL_REQUIRE(n_seqs <= 65535 * 32 && heads <= 65535, "gla_scan: too many requests or heads for one launch");
     const dim3 grid(n_seqs, heads, (value_dim + columns_a_wave - 1) / columns_a_wave);
+    if (long_portions) {
+        const int row_floats = (key_dim + 7) / 8 * 8;
+        int tile_tokens = kScanTileFloats / row_floats;
+        if (tile_tokens * columns_a_wave > kScanTileFloats) tile_tokens = kScanTileFloats / columns_a_wave;
+        if (tile_tokens > 64) tile_tokens = 64;
+        gla_scan_tiled_kernel<<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
+                                                         slots, out, heads, key_dim, value_dim, lanes_a_column, tile_tokens, q_scale);
+        return check_launch("gla_scan_tiled");
+    }
     gla_scan_kernel<<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens, slots,
                                                out, heads, key_dim, value_dim, lanes_a_column, q_scale);
     return check_launch("gla_scan");

@@ -298,9 +298,11 @@ int mll_gla_decay(const float* proj, int64_t proj_stride, int low_offset, int ra
 //   S = diag(decay_t) S + k_t v_t^T;  out[t][head] = S^T (q_t * q_scale)
 // with S = state[slots[i]][head] (float32 [key_dim][value_dim]) read at the start and written at the end.
 // q, k, v are float32 columns of proj's rows at the given offsets. A request without tokens is passed over.
+// long_portions: the kernel that brings tiles of tokens through LDS (for steps with portions of many tokens); the
+// same operations per token in the same order either way, so the same bits.
 int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset, const float* decay,
                  float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
-                 int value_dim, float q_scale, hipStream_t stream);
+                 int value_dim, float q_scale, int long_portions, hipStream_t stream);
 
 // out[t][head] = o[t][head] / rms(o[t][head]) * weight * silu(gate[t][head]) * out_scale, gate at gate_offset of
 // proj's rows; out in `dtype`, rows out_stride elements apart.

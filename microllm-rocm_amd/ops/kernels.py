@@ -1229,9 +1229,10 @@ def gla_decay(proj: torch.Tensor, low_offset: int, a2: torch.Tensor, bias: Optio
 
 def gla_scan(proj: torch.Tensor, q_offset: int, k_offset: int, v_offset: int, decay: torch.Tensor, state: torch.Tensor,
              cu_tokens: torch.Tensor, slots: torch.Tensor, n_seqs: int, heads: int, key_dim: int, value_dim: int,
-             q_scale: float) -> torch.Tensor:
+             q_scale: float, long_portions: bool = False) -> torch.Tensor:
     """The recurrence over every request's tokens of the step; ``state`` is ``[slots, heads, key_dim, value_dim]``
-    float32, read and written at ``slots``. Returns ``[tokens, heads * value_dim]`` float32."""
+    float32, read and written at ``slots``. Returns ``[tokens, heads * value_dim]`` float32. ``long_portions``: the
+    kernel that stages tiles of tokens through LDS, for steps whose requests bring many tokens (the same bits)."""
     lib = library.load()
     _device_tensor(proj, "projections", torch.float32)
     _device_tensor(decay, "decays", torch.float32)
@@ -1245,7 +1246,7 @@ def gla_scan(proj: torch.Tensor, q_offset: int, k_offset: int, v_offset: int, de
     out = torch.empty((n_tokens, heads * value_dim), dtype=torch.float32, device=proj.device)
     _check(lib.mll_gla_scan(_ptr(proj), ctypes.c_int64(proj.shape[1]), q_offset, k_offset, v_offset, _ptr(decay), _ptr(state),
                             _ptr(cu_tokens), _ptr(slots), _ptr(out), n_seqs, heads, key_dim, value_dim,
-                            ctypes.c_float(q_scale), _stream()), lib)
+                            ctypes.c_float(q_scale), int(long_portions), _stream()), lib)
     return out
 
 

@@ -28,6 +28,7 @@ class GatedLinearAttention(Mixer):
     # A step that is run twice would decay and add to the state twice: the engine, which runs a step once before it
     # captures it, saves the step's state slots before that run and puts them back (``CacheManager.save_slots``).
     graph_safe = True
+    LONG_PORTION = 8        # from this many tokens of one request in a step on, the walk stages its operands through LDS
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -90,7 +91,8 @@ class GatedLinearAttention(Mixer):
         proj = linear(x, self.in_weight, out_dtype=torch.float32)
         decay = kernels.gla_decay(proj, self.low_at, self.decay_weight, self.decay_bias, self.tau)
         o = kernels.gla_scan(proj, self.q_at, self.k_at, self.v_at, decay, cache.state, ctx.cu_tokens, ctx.slots, ctx.n_seqs,
-                             self.heads, self.key_dim, self.value_dim, self.query_scale)
+                             self.heads, self.key_dim, self.value_dim, self.query_scale,
+                             long_portions=ctx.max_count >= self.LONG_PORTION)
         return kernels.gla_gate(o, proj, self.g_at, self.norm_weight, self.eps, self.heads, self.value_dim, out_scale,
                                 self.runtime.dtype, out=out)
 

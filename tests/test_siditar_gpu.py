@@ -329,7 +329,7 @@ def test_linear_attention_walk(heads, dim, vdim, rank, tau):
     a time beside a third that starts, in slots that are not in order."""
     from microllm_rocm_amd.ops import kernels
     rng = np.random.default_rng(dim)
-    lengths = [23, 9, 4]
+    lengths = [83, 9, 4]
     keys, values = heads * dim, heads * vdim
     a2, bias, weight = rng.normal(size=(keys, rank)), rng.normal(size=keys), rng.normal(size=vdim) + 1
     columns = 2 * keys + 2 * values + rank
@@ -360,14 +360,19 @@ def test_linear_attention_walk(heads, dim, vdim, rank, tau):
         cu = np.concatenate([[0], np.cumsum([portions_of[name] for name in names])])
         proj_device = device(proj)
         decay = kernels.gla_decay(proj_device, 2 * keys + 2 * values, device(a2), device(bias), tau)
-        o = kernels.gla_scan(proj_device, 0, keys, 2 * keys, decay, state, device(cu, torch.int32),
-                             device([slot_of[name] for name in names], torch.int32), len(names), heads, dim, vdim, 0.25)
+        slots = device([slot_of[name] for name in names], torch.int32)
+        before = state.clone()      # both kernels walk the step: they must leave the same bits
+        staged = kernels.gla_scan(proj_device, 0, keys, 2 * keys, decay, before, device(cu, torch.int32), slots, len(names),
+                                  heads, dim, vdim, 0.25, long_portions=True)
+        o = kernels.gla_scan(proj_device, 0, keys, 2 * keys, decay, state, device(cu, torch.int32), slots, len(names), heads, dim,
+                             vdim, 0.25)
+        assert torch.equal(o, staged) and torch.equal(state, before)
         out = kernels.gla_gate(o, proj_device, 2 * keys + values, device(weight), 1e-5, heads, vdim, 1.5, torch.float32).cpu().numpy()
         for index, name in enumerate(names):
             got[name].append(out[cu[index]:cu[index + 1]])
             fed[name] += portions_of[name]
 
-    step({"a": 17, "b": 2})
+    step({"a": 77, "b": 2})
     step({"b": 5, "a": 1})
     step({"a": 1, "c": 4, "b": 1})
     for _ in range(4):
