@@ -33,13 +33,14 @@ __global__ void gla_decay_kernel(const float* __restrict__ proj, int64_t proj_st
 
 // One wave a (request, head, group of value channels). lane = column_in_group * lanes_a_column + r; lane r of a
 // column keeps the key channels 8 r .. 8 r + 7. A token's result is the sum over a lane's channels in order, then
-// over the column's lanes by exchanges 1, 2, 4, .. apart: both kernels below add in this order, so a request gives
-// the same bits whichever of them walks its tokens.
+// over the column's lanes in order (the lanes leave their sums in LDS and one adds them up): both kernels below add
+// in this order, so a request gives the same bits whichever of them walks its tokens.
 __global__ void __launch_bounds__(kWave)
 gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                 const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
                 const int32_t* __restrict__ slots, float* __restrict__ out, int heads, int key_dim, int value_dim,
                 int lanes_a_column, float q_scale) {
+    __shared__ float lane_sums[kWave];
     const int seq = blockIdx.x;
     const int head = blockIdx.y;
     const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
@@ -85,8 +86,14 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
             s[m] = fmaf(a[m], s[m], k[m] * v);
             partial = fmaf(s[m], q[m] * q_scale, partial);
         }
-        for (int offset = 1; offset < lanes_a_column; offset <<= 1) partial += __shfl_xor(partial, offset, kWave);
-        if (live && r == 0) out[(static_cast<int64_t>(token) * heads + head) * value_dim + column] = partial;
+        __syncthreads();      // the sums of the token before have been read
+        lane_sums[lane] = partial;
+        __syncthreads();
+        if (live && r == 0) {
+            float total = 0.0f;
+            for (int other = 0; other < lanes_a_column; ++other) total += lane_sums[lane + other];
+            out[(static_cast<int64_t>(token) * heads + head) * value_dim + column] = total;
+        }
     }
     if (!live) return;
 #pragma unroll
@@ -111,6 +118,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
                       int lanes_a_column, int tile_tokens, float q_scale) {
     __shared__ __align__(16) float buffer_even[kScanBufferFloats];
     __shared__ __align__(16) float buffer_odd[kScanBufferFloats];
+    __shared__ float lane_sums[64 * kWave];                  // of a tile's tokens (at most 64), added up after its walk
     const int seq = blockIdx.x;
     const int head = blockIdx.y;
     const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
@@ -166,6 +174,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     };
     auto walk = [&](int tile_first, const float* buffer) __attribute__((always_inline)) {
         const int count = min(tile_tokens, last - tile_first);
+#pragma unroll 4
         for (int t = 0; t < count; ++t) {
             const float* row = buffer + t * row_floats + 8 * r;
             float a[8], k[8], q[8];
@@ -182,9 +191,18 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
                 s[m] = fmaf(a[m], s[m], (valid[m] ? k[m] : 0.0f) * v);
                 partial = fmaf(s[m], q[m] * q_scale, partial);
             }
-            for (int offset = 1; offset < lanes_a_column; offset <<= 1) partial += __shfl_xor(partial, offset, kWave);
-            if (live && r == 0) out[(static_cast<int64_t>(tile_first + t) * heads + head) * value_dim + column] = partial;
+            lane_sums[t * kWave + lane] = partial;
         }
+        __syncthreads();
+        // The tile's results: a column's lanes' sums added in lane order, a result a lane, neighbours' columns by neighbours.
+        for (int result = lane; result < count * columns; result += kWave) {
+            const int t = result / columns, in_group = result % columns;
+            const int wanted = blockIdx.z * columns + in_group;
+            float total = 0.0f;
+            for (int other = 0; other < lanes_a_column; ++other) total += lane_sums[t * kWave + in_group * lanes_a_column + other];
+            if (wanted < value_dim) out[(static_cast<int64_t>(tile_first + t) * heads + head) * value_dim + wanted] = total;
+        }
+        __syncthreads();      // before the next tile's sums are written
     };
     fetch(first, buffer_even);
     for (int tile_first = first; tile_first < last;) {
