@@ -8,6 +8,8 @@
 // (all tokens at once), the walk over each request's tokens in order (the state's columns are independent, so a
 // request's head is spread over workgroups by value channel), and the norm and gate of the results. State, decays
 // and everything the walk touches are float32, whatever the engine's element type.
+#include <type_traits>
+
 #include "common.h"
 #include "microllm_hip.h"
 
@@ -84,7 +86,7 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
 #pragma unroll
         for (int m = 0; m < kStateRowsALane; ++m) {
             s[m] = fmaf(a[m], s[m], k[m] * v);
-            partial = fmaf(s[m], q[m] * q_scale, partial);
+            partial = fmaf(s[m], q[m], partial);
         }
         __syncthreads();      // the sums of the token before have been read
         lane_sums[lane] = partial;
@@ -92,7 +94,7 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
         if (live && r == 0) {
             float total = 0.0f;
             for (int other = 0; other < lanes_a_column; ++other) total += lane_sums[lane + other];
-            out[(static_cast<int64_t>(token) * heads + head) * value_dim + column] = total;
+            out[(static_cast<int64_t>(token) * heads + head) * value_dim + column] = total * q_scale;
         }
     }
     if (!live) return;
@@ -107,10 +109,11 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
 // values of its columns) from memory straight into LDS, the next tile on its way while it walks this one, and reads
 // its eight key channels of a token as two 16-byte pieces. The walk over a request's tokens stays in order, with the
 // same operations per token in the same order as above; only where the operands come from differs.
-constexpr int kScanTileFloats = 1024;                    // of each of decays, keys, queries (and at most of values) in a tile
-constexpr int kScanCalls = kScanTileFloats / kWave;      // loads of 4 bytes a lane that bring one of them
+// WIDE: rows of key channels and their places in memory are multiples of 16 bytes, and a lane's load brings 16.
+constexpr int kScanTileFloats = 2048;                    // of each of decays, keys, queries (and at most of values) in a tile
 constexpr int kScanBufferFloats = 4 * kScanTileFloats;
 
+template <bool WIDE>
 __global__ void __launch_bounds__(kWave)
 gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                       const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
@@ -118,7 +121,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
                       int lanes_a_column, int tile_tokens, float q_scale) {
     __shared__ __align__(16) float buffer_even[kScanBufferFloats];
     __shared__ __align__(16) float buffer_odd[kScanBufferFloats];
-    __shared__ float lane_sums[64 * kWave];                  // of a tile's tokens (at most 64), added up after its walk
+    __shared__ __align__(16) float lane_sums[64 * kWave];    // of a tile's tokens (at most 64), added up after its walk
     const int seq = blockIdx.x;
     const int head = blockIdx.y;
     const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
@@ -145,24 +148,39 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     for (int index = lane; index < kScanBufferFloats; index += kWave) buffer_even[index] = buffer_odd[index] = 0.0f;
     __syncthreads();
     // Which token of a tile and which channel each of this lane's loads brings (the same for every tile).
+    constexpr int kPiece = WIDE ? 4 : 1;                                  // floats a lane's load brings
+    constexpr int kScanCalls = kScanTileFloats / (kWave * kPiece);       // loads that bring one of decays, keys, queries
     int token_of[kScanCalls], channel_of[kScanCalls];
 #pragma unroll
     for (int j = 0; j < kScanCalls; ++j) {
-        const int element = j * kWave + lane;
+        const int element = (j * kWave + lane) * kPiece;
         token_of[j] = element / row_floats;
-        channel_of[j] = min(element % row_floats, key_dim - 1);
+        channel_of[j] = min(element % row_floats, key_dim - kPiece);
     }
+    bool all_valid = true;
+#pragma unroll
+    for (int m = 0; m < kStateRowsALane; ++m) all_valid = all_valid && valid[m];
+    all_valid = __all(all_valid);
     const int channels = heads * key_dim;
     const int value_calls = (tile_tokens * columns + kWave - 1) / kWave;
     auto fetch = [&](int tile_first, float* buffer) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < kScanCalls; ++j) {
-            if (j * kWave >= tile_tokens * row_floats) break;
+            if (j * kWave * (WIDE ? 4 : 1) >= tile_tokens * row_floats) break;
             const int64_t token = min(tile_first + token_of[j], last - 1);
+            constexpr int kPiece = WIDE ? 4 : 1;
             const float* row = proj + token * proj_stride + head * key_dim + channel_of[j];
-            __builtin_amdgcn_global_load_lds(decay + token * channels + head * key_dim + channel_of[j], buffer + j * kWave, 4, 0, 0);
-            __builtin_amdgcn_global_load_lds(row + k_offset, buffer + kScanTileFloats + j * kWave, 4, 0, 0);
-            __builtin_amdgcn_global_load_lds(row + q_offset, buffer + 2 * kScanTileFloats + j * kWave, 4, 0, 0);
+            const float* decays = decay + token * channels + head * key_dim + channel_of[j];
+            float* place = buffer + j * kWave * kPiece;
+            if constexpr (WIDE) {
+                __builtin_amdgcn_global_load_lds(decays, place, 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(row + k_offset, place + kScanTileFloats, 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(row + q_offset, place + 2 * kScanTileFloats, 16, 0, 0);
+            } else {
+                __builtin_amdgcn_global_load_lds(decays, place, 4, 0, 0);
+                __builtin_amdgcn_global_load_lds(row + k_offset, place + kScanTileFloats, 4, 0, 0);
+                __builtin_amdgcn_global_load_lds(row + q_offset, place + 2 * kScanTileFloats, 4, 0, 0);
+            }
         }
         for (int j = 0; j < value_calls; ++j) {
             const int element = j * kWave + lane;
@@ -172,8 +190,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
                                              buffer + 3 * kScanTileFloats + j * kWave, 4, 0, 0);
         }
     };
-    auto walk = [&](int tile_first, const float* buffer) __attribute__((always_inline)) {
-        const int count = min(tile_tokens, last - tile_first);
+    auto walk_tokens = [&](auto every_channel, int count, const float* buffer) __attribute__((always_inline)) {
 #pragma unroll 4
         for (int t = 0; t < count; ++t) {
             const float* row = buffer + t * row_floats + 8 * r;
@@ -188,19 +205,32 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
             float partial = 0.0f;
 #pragma unroll
             for (int m = 0; m < kStateRowsALane; ++m) {
-                s[m] = fmaf(a[m], s[m], (valid[m] ? k[m] : 0.0f) * v);
-                partial = fmaf(s[m], q[m] * q_scale, partial);
+                s[m] = fmaf(a[m], s[m], ((decltype(every_channel)::value || valid[m]) ? k[m] : 0.0f) * v);
+                partial = fmaf(s[m], q[m], partial);
             }
             lane_sums[t * kWave + lane] = partial;
         }
+    };
+    auto walk = [&](int tile_first, const float* buffer) __attribute__((always_inline)) {
+        const int count = min(tile_tokens, last - tile_first);
+        if (all_valid) walk_tokens(std::true_type{}, count, buffer);
+        else walk_tokens(std::false_type{}, count, buffer);
         __syncthreads();
         // The tile's results: a column's lanes' sums added in lane order, a result a lane, neighbours' columns by neighbours.
         for (int result = lane; result < count * columns; result += kWave) {
             const int t = result / columns, in_group = result % columns;
             const int wanted = blockIdx.z * columns + in_group;
+            const float* sums = lane_sums + t * kWave + in_group * lanes_a_column;
             float total = 0.0f;
-            for (int other = 0; other < lanes_a_column; ++other) total += lane_sums[t * kWave + in_group * lanes_a_column + other];
-            if (wanted < value_dim) out[(static_cast<int64_t>(tile_first + t) * heads + head) * value_dim + wanted] = total;
+            if (lanes_a_column % 4 == 0) {
+                for (int other = 0; other < lanes_a_column; other += 4) {
+                    const float4 four = *reinterpret_cast<const float4*>(sums + other);
+                    total = (((total + four.x) + four.y) + four.z) + four.w;
+                }
+            } else {
+                for (int other = 0; other < lanes_a_column; ++other) total += sums[other];
+            }
+            if (wanted < value_dim) out[(static_cast<int64_t>(tile_first + t) * heads + head) * value_dim + wanted] = total * q_scale;
         }
         __syncthreads();      // before the next tile's sums are written
     };
@@ -292,8 +322,15 @@ int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_off
         int tile_tokens = kScanTileFloats / row_floats;
         if (tile_tokens * columns_a_wave > kScanTileFloats) tile_tokens = kScanTileFloats / columns_a_wave;
         if (tile_tokens > 64) tile_tokens = 64;
-        gla_scan_tiled_kernel<<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
-                                                         slots, out, heads, key_dim, value_dim, lanes_a_column, tile_tokens, q_scale);
+        const bool wide = key_dim % 8 == 0 && proj_stride % 4 == 0 && q_offset % 4 == 0 && k_offset % 4 == 0 &&
+                          reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(decay) % 16 == 0;
+        if (wide) {
+            gla_scan_tiled_kernel<true><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
+                                                                   slots, out, heads, key_dim, value_dim, lanes_a_column, tile_tokens, q_scale);
+        } else {
+            gla_scan_tiled_kernel<false><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
+                                                                    slots, out, heads, key_dim, value_dim, lanes_a_column, tile_tokens, q_scale);
+        }
         return check_launch("gla_scan_tiled");
     }
     gla_scan_kernel<<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens, slots,

@@ -323,7 +323,7 @@ def test_mfma_bias_buckets_sink_and_far_keys():
             assert np.abs(got[-1, 0] - v[far, 0]).max() < 0.02, (far, portions_of)
 
 
-@pytest.mark.parametrize("heads,dim,vdim,rank,tau", [(3, 16, 8, 5, 4.0), (1, 40, 24, 3, 1.5), (2, 8, 72, 1, 16.0), (1, 130, 5, 2, 1.0)])
+@pytest.mark.parametrize("heads,dim,vdim,rank,tau", [(2, 16, 8, 4, 4.0), (2, 64, 128, 16, 16.0), (3, 16, 8, 5, 4.0), (1, 40, 24, 3, 1.5), (2, 8, 72, 1, 16.0), (1, 130, 5, 2, 1.0)])
 def test_linear_attention_walk(heads, dim, vdim, rank, tau):
     """Decays, the walk with carried state and the gate: two requests in one step, then both continued one token at
     a time beside a third that starts, in slots that are not in order."""
