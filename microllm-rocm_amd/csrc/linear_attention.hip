@@ -15,7 +15,11 @@
 
 namespace mll {
 
-constexpr int kStateRowsALane = 8;     // key channels a lane keeps of its column of the state
+// Key channels a lane keeps of its column of the state (ROWS below): 4 for key heads up to 256 channels, so that a
+// column is spread over more lanes and a token costs each fewer operations, 8 beyond. The choice follows the head
+// size alone, so both walk kernels make it alike.
+constexpr int kWideHeadRows = 8;
+constexpr int kUsualRows = 4;
 
 // decay[t, c] = exp(log_sigmoid(z) / tau), z = bias[c] + sum_r a2[c, r] * low[t, r]
 template <typename W>
@@ -34,9 +38,10 @@ __global__ void gla_decay_kernel(const float* __restrict__ proj, int64_t proj_st
 }
 
 // One wave a (request, head, group of value channels). lane = column_in_group * lanes_a_column + r; lane r of a
-// column keeps the key channels 8 r .. 8 r + 7. A token's result is the sum over a lane's channels in order, then
+// column keeps the key channels ROWS r .. ROWS r + ROWS - 1. A token's result is the sum over a lane's channels in order, then
 // over the column's lanes in order (the lanes leave their sums in LDS and one adds them up): both kernels below add
 // in this order, so a request gives the same bits whichever of them walks its tokens.
+template <int ROWS>
 __global__ void __launch_bounds__(kWave)
 gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                 const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
@@ -54,20 +59,20 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
     const int safe_column = live ? column : 0;
     const int slot = slots[seq];
     float* mine = state + ((static_cast<int64_t>(slot) * heads + head) * key_dim) * value_dim + safe_column;
-    float s[kStateRowsALane];
+    float s[ROWS];
 #pragma unroll
-    for (int m = 0; m < kStateRowsALane; ++m) {
-        const int i = 8 * r + m;
+    for (int m = 0; m < ROWS; ++m) {
+        const int i = ROWS * r + m;
         s[m] = i < key_dim ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
     }
     const int channels = heads * key_dim;
-    float a_next[kStateRowsALane], k_next[kStateRowsALane], q_next[kStateRowsALane], v_next;
+    float a_next[ROWS], k_next[ROWS], q_next[ROWS], v_next;
     auto fetch = [&](int token) {
         const float* row = proj + static_cast<int64_t>(token) * proj_stride;
         const float* decays = decay + static_cast<int64_t>(token) * channels + head * key_dim;
 #pragma unroll
-        for (int m = 0; m < kStateRowsALane; ++m) {
-            const int i = 8 * r + m;
+        for (int m = 0; m < ROWS; ++m) {
+            const int i = ROWS * r + m;
             const bool in = i < key_dim;
             a_next[m] = in ? decays[i] : 0.0f;
             k_next[m] = in ? row[k_offset + head * key_dim + i] : 0.0f;
@@ -77,14 +82,14 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
     };
     fetch(first);
     for (int token = first; token < last; ++token) {
-        float a[kStateRowsALane], k[kStateRowsALane], q[kStateRowsALane];
+        float a[ROWS], k[ROWS], q[ROWS];
 #pragma unroll
-        for (int m = 0; m < kStateRowsALane; ++m) a[m] = a_next[m], k[m] = k_next[m], q[m] = q_next[m];
+        for (int m = 0; m < ROWS; ++m) a[m] = a_next[m], k[m] = k_next[m], q[m] = q_next[m];
         const float v = v_next;
         if (token + 1 < last) fetch(token + 1);
         float partial = 0.0f;
 #pragma unroll
-        for (int m = 0; m < kStateRowsALane; ++m) {
+        for (int m = 0; m < ROWS; ++m) {
             s[m] = fmaf(a[m], s[m], k[m] * v);
             partial = fmaf(s[m], q[m], partial);
         }
@@ -99,21 +104,21 @@ gla_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offse
     }
     if (!live) return;
 #pragma unroll
-    for (int m = 0; m < kStateRowsALane; ++m) {
-        const int i = 8 * r + m;
+    for (int m = 0; m < ROWS; ++m) {
+        const int i = ROWS * r + m;
         if (i < key_dim) mine[static_cast<int64_t>(i) * value_dim] = s[m];
     }
 }
 
 // The same walk for portions of many tokens: a wave brings tiles of tokens (decays, keys, queries of its head, the
 // values of its columns) from memory straight into LDS, the next tile on its way while it walks this one, and reads
-// its eight key channels of a token as two 16-byte pieces. The walk over a request's tokens stays in order, with the
+// its key channels of a token in pieces of 16 bytes. The walk over a request's tokens stays in order, with the
 // same operations per token in the same order as above; only where the operands come from differs.
 // WIDE: rows of key channels and their places in memory are multiples of 16 bytes, and a lane's load brings 16.
 constexpr int kScanTileFloats = 2048;                    // of each of decays, keys, queries (and at most of values) in a tile
 constexpr int kScanBufferFloats = 4 * kScanTileFloats;
 
-template <bool WIDE>
+template <bool WIDE, int ROWS>
 __global__ void __launch_bounds__(kWave)
 gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_offset, int k_offset, int v_offset,
                       const float* __restrict__ decay, float* __restrict__ state, const int32_t* __restrict__ cu_tokens,
@@ -136,11 +141,11 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     const int row_floats = (key_dim + 7) / 8 * 8;            // a token's row of key channels in LDS
     const int slot = slots[seq];
     float* mine = state + ((static_cast<int64_t>(slot) * heads + head) * key_dim) * value_dim + safe_column;
-    float s[kStateRowsALane];
-    bool valid[kStateRowsALane];
+    float s[ROWS];
+    bool valid[ROWS];
 #pragma unroll
-    for (int m = 0; m < kStateRowsALane; ++m) {
-        const int i = 8 * r + m;
+    for (int m = 0; m < ROWS; ++m) {
+        const int i = ROWS * r + m;
         valid[m] = i < key_dim;
         s[m] = valid[m] ? mine[static_cast<int64_t>(i) * value_dim] : 0.0f;
     }
@@ -159,7 +164,7 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     }
     bool all_valid = true;
 #pragma unroll
-    for (int m = 0; m < kStateRowsALane; ++m) all_valid = all_valid && valid[m];
+    for (int m = 0; m < ROWS; ++m) all_valid = all_valid && valid[m];
     all_valid = __all(all_valid);
     const int channels = heads * key_dim;
     const int value_calls = (tile_tokens * columns + kWave - 1) / kWave;
@@ -193,18 +198,18 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     auto walk_tokens = [&](auto every_channel, int count, const float* buffer) __attribute__((always_inline)) {
 #pragma unroll 4
         for (int t = 0; t < count; ++t) {
-            const float* row = buffer + t * row_floats + 8 * r;
-            float a[8], k[8], q[8];
-            *reinterpret_cast<float4*>(a) = *reinterpret_cast<const float4*>(row);
-            *reinterpret_cast<float4*>(a + 4) = *reinterpret_cast<const float4*>(row + 4);
-            *reinterpret_cast<float4*>(k) = *reinterpret_cast<const float4*>(row + kScanTileFloats);
-            *reinterpret_cast<float4*>(k + 4) = *reinterpret_cast<const float4*>(row + kScanTileFloats + 4);
-            *reinterpret_cast<float4*>(q) = *reinterpret_cast<const float4*>(row + 2 * kScanTileFloats);
-            *reinterpret_cast<float4*>(q + 4) = *reinterpret_cast<const float4*>(row + 2 * kScanTileFloats + 4);
+            const float* row = buffer + t * row_floats + ROWS * r;
+            float a[ROWS], k[ROWS], q[ROWS];
+#pragma unroll
+            for (int piece = 0; piece < ROWS; piece += 4) {
+                *reinterpret_cast<float4*>(a + piece) = *reinterpret_cast<const float4*>(row + piece);
+                *reinterpret_cast<float4*>(k + piece) = *reinterpret_cast<const float4*>(row + kScanTileFloats + piece);
+                *reinterpret_cast<float4*>(q + piece) = *reinterpret_cast<const float4*>(row + 2 * kScanTileFloats + piece);
+            }
             const float v = buffer[3 * kScanTileFloats + t * columns + column_in_group];
             float partial = 0.0f;
 #pragma unroll
-            for (int m = 0; m < kStateRowsALane; ++m) {
+            for (int m = 0; m < ROWS; ++m) {
                 s[m] = fmaf(a[m], s[m], ((decltype(every_channel)::value || valid[m]) ? k[m] : 0.0f) * v);
                 partial = fmaf(s[m], q[m], partial);
             }
@@ -250,8 +255,8 @@ gla_scan_tiled_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
     }
     if (!live) return;
 #pragma unroll
-    for (int m = 0; m < kStateRowsALane; ++m) {
-        const int i = 8 * r + m;
+    for (int m = 0; m < ROWS; ++m) {
+        const int i = ROWS * r + m;
         if (i < key_dim) mine[static_cast<int64_t>(i) * value_dim] = s[m];
     }
 }
@@ -307,13 +312,14 @@ int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_off
                  float* state, const int32_t* cu_tokens, const int32_t* slots, float* out, int n_seqs, int heads, int key_dim,
                  int value_dim, float q_scale, int long_portions, hipStream_t stream) {
     MLL_REQUIRE(n_seqs >= 0 && heads > 0 && key_dim > 0 && value_dim > 0, "gla_scan: sizes must be positive");
-    MLL_REQUIRE(key_dim <= kStateRowsALane * kWave, "gla_scan: key heads wider than 512 are not supported");
+    MLL_REQUIRE(key_dim <= kWideHeadRows * kWave, "gla_scan: key heads wider than 512 are not supported");
     MLL_REQUIRE(q_offset >= 0 && k_offset >= 0 && v_offset >= 0 && q_offset + heads * key_dim <= proj_stride &&
                     k_offset + heads * key_dim <= proj_stride && v_offset + heads * value_dim <= proj_stride,
                 "gla_scan: a projection lies outside its row");
     if (n_seqs == 0) return 0;
+    const int rows = key_dim <= kUsualRows * kWave ? kUsualRows : kWideHeadRows;
     int lanes_a_column = 1;
-    while (lanes_a_column * kStateRowsALane < key_dim) lanes_a_column <<= 1;
+    while (lanes_a_column * rows < key_dim) lanes_a_column <<= 1;
     const int columns_a_wave = kWave / lanes_a_column;
     MLL_REQUIRE(n_seqs <= 65535 * 32 && heads <= 65535, "gla_scan: too many requests or heads for one launch");
     const dim3 grid(n_seqs, heads, (value_dim + columns_a_wave - 1) / columns_a_wave);
@@ -324,17 +330,24 @@ int mll_gla_scan(const float* proj, int64_t proj_stride, int q_offset, int k_off
         if (tile_tokens > 64) tile_tokens = 64;
         const bool wide = key_dim % 8 == 0 && proj_stride % 4 == 0 && q_offset % 4 == 0 && k_offset % 4 == 0 &&
                           reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(decay) % 16 == 0;
-        if (wide) {
-            gla_scan_tiled_kernel<true><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
-                                                                   slots, out, heads, key_dim, value_dim, lanes_a_column, tile_tokens, q_scale);
-        } else {
-            gla_scan_tiled_kernel<false><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
-                                                                    slots, out, heads, key_dim, value_dim, lanes_a_column, tile_tokens, q_scale);
-        }
+#define MLL_SCAN_TILED(WIDE, ROWS)                                                                                         \
+    gla_scan_tiled_kernel<WIDE, ROWS><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, \
+                                                                 cu_tokens, slots, out, heads, key_dim, value_dim,              \
+                                                                 lanes_a_column, tile_tokens, q_scale)
+        if (wide && rows == kUsualRows) MLL_SCAN_TILED(true, kUsualRows);
+        else if (wide) MLL_SCAN_TILED(true, kWideHeadRows);
+        else if (rows == kUsualRows) MLL_SCAN_TILED(false, kUsualRows);
+        else MLL_SCAN_TILED(false, kWideHeadRows);
+#undef MLL_SCAN_TILED
         return check_launch("gla_scan_tiled");
     }
-    gla_scan_kernel<<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens, slots,
-                                               out, heads, key_dim, value_dim, lanes_a_column, q_scale);
+    if (rows == kUsualRows) {
+        gla_scan_kernel<kUsualRows><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
+                                                               slots, out, heads, key_dim, value_dim, lanes_a_column, q_scale);
+    } else {
+        gla_scan_kernel<kWideHeadRows><<<grid, kWave, 0, stream>>>(proj, proj_stride, q_offset, k_offset, v_offset, decay, state, cu_tokens,
+                                                                  slots, out, heads, key_dim, value_dim, lanes_a_column, q_scale);
+    }
     return check_launch("gla_scan");
 }
 

@@ -12,7 +12,9 @@
 namespace mll {
 
 constexpr int kMaxStreams = 8;
-constexpr int kNormThreads = 256;
+// Threads of a row's workgroup, by the row's width alone (the order of a row's sums follows the workgroup's size, so
+// it must not follow the batch): few columns a thread keep a row of a decode step from waiting for its loads in turn.
+inline int norm_threads(int width) { return width >= 2048 ? 1024 : (width >= 1024 ? 512 : 256); }
 
 template <typename T>
 __global__ void embedding_sinusoid_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
@@ -161,10 +163,10 @@ int mll_stream_norm(float* x, const float* y, int n_parts, int64_t part_stride, 
     if (n_rows == 0) return 0;
     const size_t lds = static_cast<size_t>(width) * sizeof(float);
     if (dtype == kF32) {
-        stream_norm_kernel<float><<<n_rows, kNormThreads, lds, stream>>>(x, y, n_parts, part_stride, mix, give, take, rows, weight,
+        stream_norm_kernel<float><<<n_rows, norm_threads(width), lds, stream>>>(x, y, n_parts, part_stride, mix, give, take, rows, weight,
                                                                         eps, rms, static_cast<float*>(out), streams, width, write_x);
     } else if (dtype == kBF16) {
-        stream_norm_kernel<bf16><<<n_rows, kNormThreads, lds, stream>>>(x, y, n_parts, part_stride, mix, give, take, rows, weight,
+        stream_norm_kernel<bf16><<<n_rows, norm_threads(width), lds, stream>>>(x, y, n_parts, part_stride, mix, give, take, rows, weight,
                                                                        eps, rms, static_cast<bf16*>(out), streams, width, write_x);
     } else {
         return fail("stream_norm: unknown dtype");

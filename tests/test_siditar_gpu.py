@@ -490,3 +490,38 @@ def test_residual_stream_after_every_run(tmp_path_factory, tmp_path):
     got = np.fromfile(os.path.join(str(tmp_path), "0.layers.f32"), dtype="<f4").reshape(len(runs), 19, config["width"])
     assert len(runs) == len(plain.run_order(config)) > len(config["layers"])      # the looped layers count each time
     assert np.abs(got - np.stack(runs)).max() < 1e-4 * np.abs(np.stack(runs)).max()
+
+
+def test_command_line_and_trace_runner_as_programs(tmp_path_factory, tmp_path, capsys):
+    """The generation command line and the trace runner choose the model by its config.json like any other: greedy
+    tokens and last logits of the command line, several ways of generating, sampling with a seed, and the trace
+    runner as a program fed through a pipe."""
+    import json
+    import subprocess
+    import sys
+    from microllm_rocm_amd.cli import hf_infer
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, config, weights = model_for(tmp_path_factory, "A")
+    prompt = tokens_for(31, 13, config["vocab"])
+    expected = plain.generate_greedy(config, weights, prompt, 6)
+    base = ["--model", folder, "--tokens", ",".join(map(str, prompt)), "--new-tokens", "6", "--dtype", "float32"]
+
+    def run(*more):
+        capsys.readouterr()
+        assert hf_infer.main(base + list(more)) == 0
+        return json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+
+    logits_path = tmp_path / "last.f32"
+    report = run("--logits-output", str(logits_path))
+    assert report["architecture"] == "Siditar" and report["generated_tokens"] == expected
+    assert row_errors(np.fromfile(logits_path, dtype="<f4")[None], plain.forward(config, weights, prompt)[-1:]).max() < F32_BOUND
+    for more in (["--use-cache", "false"], ["--cache-prefill-mode", "token"], ["--batch", "2", "--batch-argmax-mode", "host"]):
+        assert run(*more)["generated_tokens"] == expected, more
+    sampled = [run("--temperature", "0.9", "--sample-top-k", "5", "--seed", "7")["generated_tokens"] for _ in range(2)]
+    assert sampled[0] == sampled[1] and len(sampled[0]) == 6
+    steps = portions("p", prompt + expected, [5, 2, 1])
+    result = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out",
+                             str(tmp_path / "trace"), "--max-tokens", "64"], input=to_lines(steps), capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stderr
+    assert [line for line in result.stdout.splitlines() if line.startswith("done")] == [f"done {step['step']}" for step in steps]
+    check_against_plain(steps, tmp_path / "trace", {"p": prompt + expected}, config, weights, "float32")
