@@ -202,8 +202,6 @@ class SiditarConfig:
         _positive(self.vocab, "vocab")
         _positive(self.width, "width")
         _positive(self.norm_eps, "norm.eps")
-        if self.width % 2 != 0:
-            raise ConfigError("width must be even: the position vector comes in pairs of sine and cosine")
         if self.streams is not None and not 1 <= self.streams <= 8:
             raise ConfigError("streams must lie between 1 and 8")
         if self.loop is not None:

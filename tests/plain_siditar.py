@@ -27,10 +27,9 @@ def position_waves(count: int, width: int, first: int = 0) -> np.ndarray:
     """Row p: entry 2i is sin(p / 10000^(2i / width)), entry 2i + 1 the cosine of the same angle."""
     out = np.zeros((count, width))
     for row in range(count):
-        for pair in range(width // 2):
-            angle = (first + row) * 10000.0 ** (-2.0 * pair / width)
-            out[row, 2 * pair] = math.sin(angle)
-            out[row, 2 * pair + 1] = math.cos(angle)
+        for column in range(width):
+            angle = (first + row) * 10000.0 ** (-2.0 * (column // 2) / width)
+            out[row, column] = math.cos(angle) if column % 2 else math.sin(angle)
     return out
 
 

@@ -35,10 +35,10 @@ TINY_B = SiditarConfig(
         _layer(BiasAttentionConfig(heads=2, kv_heads=2, dim=32, vdim=12, scale=0.15, bias_max=64, temp_coef=0.0, temp_every=3, bias_rows=4),
                LinearAttentionConfig(heads=5, dim=8, vdim=8, tau=2.0, decay_rank=8), (1.1, 1.4), DenseMlpConfig(64, 0.75)),
     ))
-# One stream that still goes through its connection weights; a loop over the last layer alone, twice; no feed-forward
+# One stream that still goes through its connection weights; a width that is no multiple of 4; a loop over the last layer alone, twice; no feed-forward
 # in the first layer.
 TINY_C = SiditarConfig(
-    vocab=130, width=48, norm_eps=1e-5, streams=1, loop=LoopConfig(1, 2, 2),
+    vocab=130, width=50, norm_eps=1e-5, streams=1, loop=LoopConfig(1, 2, 2),
     layers=(
         _layer(BiasAttentionConfig(heads=2, kv_heads=2, dim=12, vdim=20, scale=0.3, bias_max=17, temp_coef=0.5, temp_every=4, bias_rows=8),
                LinearAttentionConfig(heads=4, dim=12, vdim=12, tau=3.0, decay_rank=2), (1.0, 0.6), None),

@@ -81,7 +81,7 @@ def device(array, dtype=torch.float32):
     return torch.as_tensor(np.asarray(array), dtype=dtype).cuda().contiguous()
 
 
-@pytest.mark.parametrize("width,first", [(64, 0), (50, 1000), (6, 7)])
+@pytest.mark.parametrize("width,first", [(64, 0), (50, 1000), (6, 7), (37, 3)])
 def test_embedding_adds_sine_and_cosine(width, first):
     from microllm_rocm_amd.ops import kernels
     rng = np.random.default_rng(0)
