@@ -242,9 +242,9 @@ int mll_paged_attention_prefill_extra(const void* q, const void* k_cache, const 
 // ---- several copies of the residual stream, a norm with a mean, a sinusoidal position vector ----------------
 
 // out[t, :] = table[ids[t], :] + wave(positions[t]) in float32, where entry 2i of the wave is
-// sin(p * base^(-2i / width)) and entry 2i + 1 the cosine of the same angle (the angle in float64).
-int mll_embedding_sinusoid(const void* table, int table_dtype, const int32_t* ids, const int32_t* positions, float* out,
-                           int n_tokens, int width, int vocab, double base, hipStream_t stream);
+// sin(p * rates[i]) and entry 2i + 1 the cosine of the same angle (the angle in float64; rates: (width + 1) / 2 doubles).
+int mll_embedding_sinusoid(const void* table, int table_dtype, const int32_t* ids, const int32_t* positions,
+                           const double* rates, float* out, int n_tokens, int width, int vocab, hipStream_t stream);
 
 // out[t, c, :] = in[t, :] for every copy c: float32 [n_tokens][copies][width].
 int mll_stream_copies(const float* in, float* out, int n_tokens, int width, int copies, hipStream_t stream);

@@ -18,8 +18,8 @@ inline int norm_threads(int width) { return width >= 2048 ? 1024 : (width >= 102
 
 template <typename T>
 __global__ void embedding_sinusoid_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                                          const int32_t* __restrict__ positions, float* __restrict__ out, int width,
-                                          int vocab, double base) {
+                                          const int32_t* __restrict__ positions, const double* __restrict__ rates,
+                                          float* __restrict__ out, int width, int vocab) {
     const int token = blockIdx.x;
     const int id = ids[token];
     const bool valid = id >= 0 && id < vocab;
@@ -27,9 +27,8 @@ __global__ void embedding_sinusoid_kernel(const T* __restrict__ table, const int
     const T* row = table + static_cast<int64_t>(valid ? id : 0) * width;
     float* to = out + static_cast<int64_t>(token) * width;
     for (int column = threadIdx.x; column < width; column += blockDim.x) {
-        // entry 2i: sin(p * base^(-2i / width)), entry 2i + 1: cos of the same angle; the angle in float64
-        const int pair = column / 2;
-        const double angle = position * pow(base, -2.0 * static_cast<double>(pair) / static_cast<double>(width));
+        // entry 2i: sin(p * rates[i]), entry 2i + 1: cos of the same angle; the angle in float64
+        const double angle = position * rates[column / 2];
         const float wave = static_cast<float>((column & 1) ? cos(angle) : sin(angle));
         to[column] = valid ? to_float(row[column]) + wave : __builtin_nanf("");
     }
@@ -128,16 +127,16 @@ using namespace mll;
 
 extern "C" {
 
-int mll_embedding_sinusoid(const void* table, int table_dtype, const int32_t* ids, const int32_t* positions, float* out,
-                           int n_tokens, int width, int vocab, double base, hipStream_t stream) {
-    MLL_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0 && base > 0.0, "embedding_sinusoid: sizes must be positive");
+int mll_embedding_sinusoid(const void* table, int table_dtype, const int32_t* ids, const int32_t* positions,
+                           const double* rates, float* out, int n_tokens, int width, int vocab, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && width > 0 && vocab > 0 && rates != nullptr, "embedding_sinusoid: sizes must be positive");
     if (n_tokens == 0) return 0;
     if (table_dtype == kF32) {
-        embedding_sinusoid_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, positions, out,
-                                                                      width, vocab, base);
+        embedding_sinusoid_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(table), ids, positions, rates,
+                                                                      out, width, vocab);
     } else if (table_dtype == kBF16) {
-        embedding_sinusoid_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, positions, out,
-                                                                     width, vocab, base);
+        embedding_sinusoid_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(table), ids, positions, rates,
+                                                                     out, width, vocab);
     } else {
         return fail("embedding_sinusoid: unknown table dtype");
     }

@@ -1026,19 +1026,21 @@ def measured_peaks(device: Optional[torch.device] = None, read_bytes: int = 4 <<
 
 
 # ---- several copies of the residual stream; a norm with a mean; a sinusoidal position vector --------------------
-def embedding_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, base: float) -> torch.Tensor:
-    """``table[ids] + wave(positions)`` in float32; entry 2i of the wave is ``sin(p * base^(-2i / width))``, entry
-    2i + 1 the cosine of the same angle."""
+def embedding_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, rates: torch.Tensor) -> torch.Tensor:
+    """``table[ids] + wave(positions)`` in float32; entry 2i of the wave is ``sin(p * rates[i])``, entry 2i + 1 the
+    cosine of the same angle (``rates``: float64, one per pair of columns)."""
     lib = library.load()
     _device_tensor(table, "embedding table")
     _device_tensor(ids, "token ids", torch.int32)
     _device_tensor(positions, "positions", torch.int32)
+    _device_tensor(rates, "rates of the position waves", torch.float64)
     _need(table.dim() == 2 and ids.dim() == 1 and positions.shape == ids.shape,
           "embedding_sinusoid takes a [vocab, width] table and [tokens] ids and positions")
     vocab, width = table.shape
+    _need(tuple(rates.shape) == ((width + 1) // 2,), "one rate per pair of columns")
     out = torch.empty((ids.shape[0], width), dtype=torch.float32, device=table.device)
-    _check(lib.mll_embedding_sinusoid(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(positions), _ptr(out),
-                                      ids.shape[0], width, vocab, ctypes.c_double(base), _stream()), lib)
+    _check(lib.mll_embedding_sinusoid(_ptr(table), _code(table.dtype), _ptr(ids), _ptr(positions), _ptr(rates), _ptr(out),
+                                      ids.shape[0], width, vocab, _stream()), lib)
     return out
 
 

@@ -106,6 +106,9 @@ class SinusoidTokenEmbedding(Part):
         self.vocab = int(spec.params["vocab_size"])
         self.width = int(spec.params["hidden_size"])
         self.base = float(spec.params.get("base", 10000.0))
+        # base^(-2i / width) for every pair of columns, in float64 as the angles are
+        pairs = torch.arange((self.width + 1) // 2, dtype=torch.float64)
+        self.rates = (self.base ** (-2.0 * pairs / self.width)).to(runtime.device)
         self.table: Optional[torch.Tensor] = None
 
     def tensors(self):
@@ -115,7 +118,7 @@ class SinusoidTokenEmbedding(Part):
         self.table = tensors[self.name("weight")]
 
     def forward(self, ctx) -> torch.Tensor:
-        return kernels.embedding_sinusoid(self.table, ctx.tokens, ctx.positions, self.base)
+        return kernels.embedding_sinusoid(self.table, ctx.tokens, ctx.positions, self.rates)
 
     def bytes_read(self, rows: int, context: int) -> int:
         return rows * self.width * self.table.element_size()

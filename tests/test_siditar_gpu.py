@@ -88,7 +88,8 @@ def test_embedding_adds_sine_and_cosine(width, first):
     table = rng.normal(size=(17, width)).astype(np.float32)
     ids = rng.integers(0, 17, size=9)
     positions = np.arange(first, first + 9)
-    got = kernels.embedding_sinusoid(device(table), device(ids, torch.int32), device(positions, torch.int32), 10000.0)
+    rates = device(10000.0 ** (-2.0 * np.arange((width + 1) // 2) / width), torch.float64)
+    got = kernels.embedding_sinusoid(device(table), device(ids, torch.int32), device(positions, torch.int32), rates)
     want = table[ids] + plain.position_waves(9, width, first)
     assert np.abs(got.cpu().numpy() - want).max() < 1e-6
 
