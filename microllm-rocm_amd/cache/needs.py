@@ -149,6 +149,39 @@ class PagedKeyValueNeed(CacheNeed):
         return PagedBinding(self, owned, group, k, v)
 
 
+# ---- one latent row a position, in plain pages -------------------------------------------------------------------------
+@dataclass(frozen=True)
+class PagedLatentNeed(CacheNeed):
+    """One row of ``width`` elements a position, ``[page, position, width]``: what an attention keeps whose keys and
+    values are projections of one cached vector (a latent and whatever rides with it, e.g. a rotated key part)."""
+    width: int
+    window: Optional[int] = None
+    paged = True
+
+    def check_page_size(self, page_size: int) -> None:
+        if page_size <= 0:
+            raise ValueError("page_size must be positive")
+
+    def allocate_pages(self, num_pages, page_size, dtype, device):
+        return torch.zeros((num_pages, page_size, self.width), dtype=dtype, device=device)
+
+    def bytes_per_position(self, dtype):
+        return self.width * _element_size(dtype)
+
+    def bind(self, group, storage, owned):
+        return LatentBinding(self, owned, group, storage)
+
+
+@dataclass
+class LatentBinding(Binding):
+    """What a mixer gets for latent rows in pages: its entry's page array and its group."""
+    group: int = 0
+    rows: Optional[torch.Tensor] = None
+
+    def tensors(self):
+        return [self.rows] if self.rows is not None else []
+
+
 # ---- per-request state of fixed size -------------------------------------------------------------
 @dataclass(frozen=True)
 class StateNeed(CacheNeed):

@@ -310,4 +310,77 @@ int mll_gla_gate(const float* o, const float* proj, int64_t proj_stride, int gat
                  void* out, int64_t out_stride, int dtype, int n_tokens, int heads, int value_dim, float out_scale,
                  hipStream_t stream);
 
+// ---- attention through latents (csrc/latent_attention.hip) ----------------------------------------------------
+
+// proj[t] holds, in float32, the queries' down projection at q_at (q_rank wide) and the keys' and values' at kv_at
+// (kv_rank, then rot_dim). q_latent[t] = proj / rms * q_weight in `dtype`. With slot_mapping (null: the layer stores
+// nothing): the first kv_rank entries / rms * kv_weight and the last rot_dim turned by the split-half rule with
+// cos_sin [t][rot_dim / 2][2] go to slot slot_mapping[t] (negative: not stored) of `pages` [slot][kv_rank + rot_dim],
+// or, with tiled_page_size > 0, of k_pages and v_pages (one kv head of kv_rank + rot_dim dims, cache_layout.h): the
+// same row as key and as value.
+int mll_latent_prepare(const float* proj, int64_t proj_stride, int q_at, int q_rank, const float* q_weight, int kv_at,
+                       int kv_rank, int rot_dim, const float* kv_weight, float eps, const float* cos_sin,
+                       const int32_t* slot_mapping, void* q_latent, void* pages, void* k_pages, void* v_pages,
+                       int tiled_page_size, int dtype, int n_tokens, hipStream_t stream);
+
+// q: float32 [t][head][dim | rot_dim]. q_full [t][head][kv_rank | rot_dim] in `dtype` gets the rotated part turned;
+// `folded` ([head][t][kv_rank], nullable) is copied in front of it; `flat_out` ([head][t][dim], nullable) receives
+// the unrotated part.
+int mll_latent_query(const float* q, int n_tokens, int heads, int dim, int rot_dim, int kv_rank, const float* cos_sin,
+                     const void* folded, void* flat_out, void* q_full, int dtype, hipStream_t stream);
+
+// out[t][h][o] = sum_i x[t][h][i] * w[h][i][o] (* sigmoid(gate[t][h * n_out + o]) with gate, float32 rows gate_stride
+// apart), sums float32 in ascending i. Strides in elements. Built for (x, w, out) = (f32, f32, f32), (f32, bf16, bf16),
+// (bf16, bf16, bf16), (f32, bf16, f32).
+int mll_head_product(const void* x, int x_dtype, int64_t x_token_stride, int64_t x_head_stride, const void* w, int w_dtype,
+                     void* out, int out_dtype, int64_t out_token_stride, int64_t out_head_stride, const float* gate,
+                     int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream);
+
+// For every token and head: softmax over the keys j in (p - window, p] (window <= 0: all j <= p) of
+// (q_full[t][h] . pages[slot_j]) * scale, out[t][h] = sum_j weight_j pages[slot_j][:kv_rank]. A token whose
+// seq_of_token is negative is skipped. The order of every sum depends on p and the window alone.
+int mll_latent_attention(const void* q_full, const void* pages, const int32_t* block_table, int table_width,
+                         const int32_t* seq_of_token, const int32_t* positions, void* out, int64_t out_token_stride,
+                         int64_t out_head_stride, int dtype, int n_tokens, int heads, int kv_rank, int rot_dim, int page_size,
+                         int window, float scale, hipStream_t stream);
+
+// ---- a recurrent block with a gated linear recurrence (csrc/recurrent.hip) ----------------------------------------
+
+// u[t][c] = conv_bias[c] + sum_j taps[c][j] * input(t - (n_taps - 1 - j), c), input = proj[.][x_at + c] + x_bias[c] for
+// the step's tokens of the same request, the request's kept inputs (kept [slot][n_taps - 1][width], newest last)
+// before them. Biases nullable. taps in taps_dtype.
+int mll_rglru_conv(const float* proj, int64_t proj_stride, int x_at, const float* x_bias, const void* taps, int taps_dtype,
+                   const float* conv_bias, const float* kept, const int32_t* seq_of_token, const int32_t* cu_tokens,
+                   const int32_t* slots, float* u, int n_tokens, int width, int n_taps, hipStream_t stream);
+
+// Per request and channel, over the request's tokens in order: r = sigmoid(gates[t][b][c'] + r_bias), i =
+// sigmoid(gates[t][b][size + c'] + i_bias) (gates: float32 [t][blocks][2 * size]), a = exp(-decay_scale * r *
+// softplus(lam)), S = a S + sqrt(1 - a^2) * i * u; out[t][c] = S * gelu_tanh(proj[t][y_at + c] + y_bias[c]) in `dtype`.
+// S = state[slot][c] is read first and written last, and `kept` receives the convolution's newest inputs.
+int mll_rglru_scan(const float* proj, int64_t proj_stride, int x_at, const float* x_bias, int y_at, const float* y_bias,
+                   const float* u, const float* gates, const float* r_bias, const float* i_bias, const float* lam,
+                   float decay_scale, float* state, float* kept, const int32_t* cu_tokens, const int32_t* slots, void* out,
+                   int dtype, int n_seqs, int width, int blocks, int n_taps, hipStream_t stream);
+
+// ---- a mixture of experts (csrc/moe.hip) ------------------------------------------------------------------------
+
+// ids[t][n], weights[t][n] for n < top: the experts with the largest scores (sigmoid, or softmax over the experts)
+// of z[t][0 .. experts), ties to the lower index; weights are the scores, divided by their sum with renormalize.
+// shared_at >= 0: shared_gate[t] = sigmoid(z[t][shared_at]).
+int mll_moe_route(const float* z, int64_t z_stride, int n_tokens, int experts, int top, int softmax_scores, int renormalize,
+                  int shared_at, int32_t* ids, float* weights, float* shared_gate, hipStream_t stream);
+
+// act[t * top + n] = silu(Wg_e xs) * (Wu_e xs), e = ids[t][n], xs = x[t] * weights[t][n] rounded to `dtype`
+// (weight_on_input) or x[t]; gate_up [experts][2 * ff][width] with the gate rows first.
+int mll_moe_gate_up(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, void* act,
+                    int dtype, int n_tokens, int width, int ff, int weight_on_input, hipStream_t stream);
+
+// out[n][t] = Wd_e act[t * top + n] (* weights[t][n] unless weight_on_input): float32 [top][n_tokens][width].
+int mll_moe_down(const void* act, const int32_t* ids, const float* weights, int top, const void* down, float* out, int dtype,
+                 int n_tokens, int width, int ff, int weight_on_input, hipStream_t stream);
+
+// out[t] = factor[t] * (in[0][t] + in[1][t] + ...), float32; parts part_stride elements apart.
+int mll_scale_rows(const float* in, int n_parts, int64_t part_stride, const float* factor, float* out, int n_tokens, int width,
+                   hipStream_t stream);
+
 }  // extern "C"

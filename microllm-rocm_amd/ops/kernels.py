@@ -1270,3 +1270,237 @@ def gla_gate(o: torch.Tensor, proj: torch.Tensor, gate_offset: int, weight: torc
                             ctypes.c_void_p(out.data_ptr()), ctypes.c_int64(max(out.stride(0), heads * value_dim)), _code(out_dtype),
                             n_tokens, heads, value_dim, ctypes.c_float(out_scale), _stream()), lib)
     return out
+
+
+# ---- attention through latents -----------------------------------------------------------------------------------
+def latent_prepare(proj: torch.Tensor, q_at: int, q_rank: int, q_weight: torch.Tensor, kv_at: int, kv_rank: int, rot_dim: int,
+                   kv_weight: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
+                   slot_mapping: Optional[torch.Tensor], out_dtype: torch.dtype, pages: Optional[torch.Tensor] = None,
+                   k_pages: Optional[torch.Tensor] = None, v_pages: Optional[torch.Tensor] = None,
+                   tiled_page_size: int = 0) -> torch.Tensor:
+    """The norms of a token's two latents from its float32 down projections ``proj`` ``[tokens, columns]``; returns the
+    queries' normed latent ``[tokens, q_rank]``. With ``slot_mapping`` the keys' normed latent and the turned key
+    part go into ``pages`` ``[page, position, kv_rank + rot_dim]`` or, with ``tiled_page_size``, into key and value
+    pages of ``cache.layout`` (one kv head of ``kv_rank + rot_dim`` dims, the same row in both)."""
+    lib = library.load()
+    _device_tensor(proj, "down projections", torch.float32)
+    _need(proj.dim() == 2 and 0 <= q_at and q_at + q_rank <= proj.shape[1], "the queries' latent lies outside the projections' rows")
+    _device_tensor(q_weight, "query latent norm weight", torch.float32)
+    _need(tuple(q_weight.shape) == (q_rank,), "the queries' norm weight must match their latent")
+    n_tokens = proj.shape[0]
+    if slot_mapping is not None:
+        _need(0 <= kv_at and kv_at + kv_rank + rot_dim <= proj.shape[1], "the keys' latent lies outside the projections' rows")
+        _device_tensor(slot_mapping, "slot mapping", torch.int32)
+        _device_tensor(kv_weight, "latent norm weight", torch.float32)
+        _device_tensor(cos_sin, "cos/sin table", torch.float32)
+        _need(slot_mapping.shape[0] >= n_tokens and tuple(kv_weight.shape) == (kv_rank,), "a slot a token and a weight a latent channel")
+        _need(tuple(cos_sin.shape) == (n_tokens, rot_dim // 2, 2) and rot_dim % 2 == 0, "the cos/sin table must be [tokens, rot_dim / 2, 2]")
+        if tiled_page_size:
+            _check_pages(k_pages, v_pages, out_dtype, 1, kv_rank + rot_dim, tiled_page_size)
+        else:
+            _device_tensor(pages, "latent pages", out_dtype)
+            _need(pages.dim() == 3 and pages.shape[2] == kv_rank + rot_dim, "latent pages are [page, position, kv_rank + rot_dim]")
+    q_latent = torch.empty((n_tokens, q_rank), dtype=out_dtype, device=proj.device)
+    _check(lib.mll_latent_prepare(_ptr(proj), ctypes.c_int64(proj.shape[1]), q_at, q_rank, _ptr(q_weight), kv_at, kv_rank, rot_dim,
+                                  _ptr(kv_weight), ctypes.c_float(eps), _ptr(cos_sin), _ptr(slot_mapping), _ptr(q_latent),
+                                  _ptr(pages), _ptr(k_pages), _ptr(v_pages), int(tiled_page_size), _code(out_dtype), n_tokens,
+                                  _stream()), lib)
+    return q_latent
+
+
+def latent_query(q: torch.Tensor, heads: int, dim: int, rot_dim: int, kv_rank: int, cos_sin: torch.Tensor, q_full: torch.Tensor,
+                 folded: Optional[torch.Tensor] = None, want_flat: bool = False) -> Optional[torch.Tensor]:
+    """``q`` float32 ``[tokens, heads * (dim + rot_dim)]``: the turned rotated parts go behind the folded parts in
+    ``q_full`` ``[tokens, heads * (kv_rank + rot_dim)]``; ``folded`` ``[heads, tokens, kv_rank]`` is copied in front;
+    with ``want_flat`` the unrotated parts are returned as ``[heads, tokens, dim]`` in ``q_full``'s dtype."""
+    lib = library.load()
+    _device_tensor(q, "queries", torch.float32)
+    n_tokens = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] == heads * (dim + rot_dim), "queries are [tokens, heads * (dim + rot_dim)]")
+    _device_tensor(cos_sin, "cos/sin table", torch.float32)
+    _need(tuple(cos_sin.shape) == (n_tokens, rot_dim // 2, 2) and rot_dim % 2 == 0, "the cos/sin table must be [tokens, rot_dim / 2, 2]")
+    _device_tensor(q_full, "folded queries")
+    _need(tuple(q_full.shape) == (n_tokens, heads * (kv_rank + rot_dim)), "folded queries are [tokens, heads * (kv_rank + rot_dim)]")
+    if folded is not None:
+        _device_tensor(folded, "folded parts", q_full.dtype)
+        _need(tuple(folded.shape) == (heads, n_tokens, kv_rank), "folded parts are [heads, tokens, kv_rank]")
+    flat = torch.empty((heads, n_tokens, dim), dtype=q_full.dtype, device=q.device) if want_flat else None
+    _check(lib.mll_latent_query(_ptr(q), n_tokens, heads, dim, rot_dim, kv_rank, _ptr(cos_sin), _ptr(folded), _ptr(flat), _ptr(q_full),
+                                _code(q_full.dtype), _stream()), lib)
+    return flat
+
+
+HEAD_PRODUCT_TYPES = {(torch.float32, torch.float32, torch.float32), (torch.float32, torch.bfloat16, torch.bfloat16),
+                      (torch.bfloat16, torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16, torch.float32)}
+
+
+def head_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t, h, o] = sum_i x[t, h, i] * weight[h, i, o]``, times ``sigmoid(gate[t, h * n_out + o])`` with ``gate``
+    (float32 rows). ``x`` ``[tokens, heads, n_in]`` and ``out`` ``[tokens, heads, n_out]`` may be views with strides of
+    their own over tokens and heads (unit stride along the last axis); the weight is contiguous."""
+    lib = library.load()
+    _device_tensor(weight, "per-head weight")
+    _need(weight.dim() == 3, "the weight is [heads, n_in, n_out]")
+    heads, n_in, n_out = weight.shape
+    _need(x.is_cuda and x.dim() == 3 and x.shape[1:] == (heads, n_in) and x.stride(2) == 1, "x is [tokens, heads, n_in] with unit stride along n_in")
+    n_tokens = x.shape[0]
+    _need(out.is_cuda and tuple(out.shape) == (n_tokens, heads, n_out) and out.stride(2) == 1, "out is [tokens, heads, n_out] with unit stride along n_out")
+    _need((x.dtype, weight.dtype, out.dtype) in HEAD_PRODUCT_TYPES, f"head_product is not built for {x.dtype}, {weight.dtype}, {out.dtype}")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape == (n_tokens, heads * n_out) and gate.stride(1) == 1,
+              "the gate is float32 [tokens, heads * n_out] with unit column stride")
+        gate_stride = gate.stride(0)
+    _check(lib.mll_head_product(ctypes.c_void_p(x.data_ptr()), _code(x.dtype), ctypes.c_int64(x.stride(0)), ctypes.c_int64(x.stride(1)),
+                                _ptr(weight), _code(weight.dtype), ctypes.c_void_p(out.data_ptr()), _code(out.dtype),
+                                ctypes.c_int64(out.stride(0)), ctypes.c_int64(out.stride(1)),
+                                ctypes.c_void_p(gate.data_ptr() if gate is not None else 0), ctypes.c_int64(gate_stride),
+                                n_tokens, heads, n_in, n_out, _stream()), lib)
+    return out
+
+
+def latent_attention(q_full: torch.Tensor, pages: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
+                     positions: torch.Tensor, scale: float, window: int, heads: int, kv_rank: int, rot_dim: int) -> torch.Tensor:
+    """Attention of folded queries ``[tokens, heads * (kv_rank + rot_dim)]`` over latent pages ``[page, position, kv_rank
+    + rot_dim]``; returns the weighted latents ``[tokens, heads, kv_rank]``."""
+    lib = library.load()
+    _device_tensor(q_full, "folded queries")
+    n_tokens = q_full.shape[0]
+    width = kv_rank + rot_dim
+    _need(q_full.dim() == 2 and q_full.shape[1] == heads * width, "folded queries are [tokens, heads * (kv_rank + rot_dim)]")
+    _device_tensor(pages, "latent pages", q_full.dtype)
+    _need(pages.dim() == 3 and pages.shape[2] == width, "latent pages are [page, position, kv_rank + rot_dim]")
+    _device_tensor(block_table, "block table", torch.int32)
+    _device_tensor(seq_of_token, "request of every token", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    _need(block_table.dim() == 2 and seq_of_token.shape[0] >= n_tokens and positions.shape[0] >= n_tokens,
+          "a block table [requests, width] and a request and a position for every token")
+    out = torch.empty((n_tokens, heads, kv_rank), dtype=q_full.dtype, device=q_full.device)
+    _check(lib.mll_latent_attention(_ptr(q_full), _ptr(pages), _ptr(block_table), block_table.shape[1], _ptr(seq_of_token),
+                                    _ptr(positions), _ptr(out), ctypes.c_int64(heads * kv_rank), ctypes.c_int64(kv_rank),
+                                    _code(q_full.dtype), n_tokens, heads, kv_rank, rot_dim, pages.shape[1], int(window),
+                                    ctypes.c_float(scale), _stream()), lib)
+    return out
+
+
+# ---- a recurrent block with a gated linear recurrence -----------------------------------------------------------------
+def rglru_conv(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], taps: torch.Tensor, conv_bias: Optional[torch.Tensor],
+               kept: torch.Tensor, seq_of_token: torch.Tensor, cu_tokens: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """The causal convolution per channel over ``proj[:, x_at : x_at + width] + x_bias``, continued from the inputs
+    each request kept (``kept``: float32 ``[slots, taps - 1, width]``); float32 ``[tokens, width]``."""
+    lib = library.load()
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(taps, "taps")
+    _need(proj.dim() == 2 and taps.dim() == 2, "projections [tokens, columns] and taps [width, taps]")
+    width, n_taps = taps.shape
+    _need(0 <= x_at and x_at + width <= proj.shape[1], "the convolution's input lies outside the projections' rows")
+    for name, bias in (("input bias", x_bias), ("convolution bias", conv_bias)):
+        if bias is not None:
+            _device_tensor(bias, name, torch.float32)
+            _need(tuple(bias.shape) == (width,), f"one {name} a channel")
+    _device_tensor(kept, "kept inputs", torch.float32)
+    _need(kept.dim() == 3 and tuple(kept.shape[1:]) == (n_taps - 1, width), "kept inputs are [slots, taps - 1, width]")
+    n_tokens = proj.shape[0]
+    for name, tensor in (("request of every token", seq_of_token), ("token offsets", cu_tokens), ("state slots", slots)):
+        _device_tensor(tensor, name, torch.int32)
+    _need(seq_of_token.shape[0] >= n_tokens, "a request for every token")
+    u = torch.empty((n_tokens, width), dtype=torch.float32, device=proj.device)
+    _check(lib.mll_rglru_conv(_ptr(proj), ctypes.c_int64(proj.shape[1]), x_at, _ptr(x_bias), _ptr(taps), _code(taps.dtype),
+                              _ptr(conv_bias), _ptr(kept), _ptr(seq_of_token), _ptr(cu_tokens), _ptr(slots), _ptr(u), n_tokens, width,
+                              n_taps, _stream()), lib)
+    return u
+
+
+def rglru_scan(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], y_at: int, y_bias: Optional[torch.Tensor],
+               u: torch.Tensor, gates: torch.Tensor, r_bias: Optional[torch.Tensor], i_bias: Optional[torch.Tensor],
+               lam: torch.Tensor, decay_scale: float, state: torch.Tensor, kept: torch.Tensor, cu_tokens: torch.Tensor,
+               slots: torch.Tensor, n_seqs: int, blocks: int, n_taps: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """The gated linear recurrence over every request's tokens of the step, times the gated branch; ``state`` float32
+    ``[slots, width]`` and ``kept`` ``[slots, taps - 1, width]`` are read and written at ``slots``. Returns
+    ``[tokens, width]`` in ``out_dtype``."""
+    lib = library.load()
+    _device_tensor(proj, "projections", torch.float32)
+    _device_tensor(u, "convolution output", torch.float32)
+    _device_tensor(gates, "gates", torch.float32)
+    _device_tensor(lam, "decay parameter", torch.float32)
+    _device_tensor(state, "state", torch.float32)
+    _device_tensor(kept, "kept inputs", torch.float32)
+    n_tokens, width = u.shape
+    _need(proj.shape[0] == n_tokens and max(x_at, y_at) + width <= proj.shape[1], "the branches lie outside the projections' rows")
+    _need(tuple(gates.shape) == (n_tokens, 2 * width) and tuple(lam.shape) == (width,) and width % blocks == 0, "gates are [tokens, 2 * width]")
+    _need(state.dim() == 2 and state.shape[1] == width and kept.dim() == 3 and tuple(kept.shape[1:]) == (n_taps - 1, width)
+          and kept.shape[0] == state.shape[0], "state is [slots, width], kept inputs [slots, taps - 1, width]")
+    for name, bias in (("input bias", x_bias), ("branch bias", y_bias), ("gate bias", r_bias), ("gate bias", i_bias)):
+        if bias is not None:
+            _device_tensor(bias, name, torch.float32)
+            _need(bias.numel() == width, f"one {name} a channel")
+    _device_tensor(cu_tokens, "token offsets", torch.int32)
+    _device_tensor(slots, "state slots", torch.int32)
+    _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
+    out = torch.empty((n_tokens, width), dtype=out_dtype, device=u.device)
+    _check(lib.mll_rglru_scan(_ptr(proj), ctypes.c_int64(proj.shape[1]), x_at, _ptr(x_bias), y_at, _ptr(y_bias), _ptr(u), _ptr(gates),
+                              _ptr(r_bias), _ptr(i_bias), _ptr(lam), ctypes.c_float(decay_scale), _ptr(state), _ptr(kept),
+                              _ptr(cu_tokens), _ptr(slots), _ptr(out), _code(out_dtype), n_seqs, width, blocks, n_taps, _stream()), lib)
+    return out
+
+
+# ---- a mixture of experts ------------------------------------------------------------------------------------------
+def moe_route(z: torch.Tensor, experts: int, top: int, softmax_scores: bool = False, renormalize: bool = False,
+              shared_at: int = -1):
+    """The ``top`` experts of every token from router logits ``z`` float32 ``[tokens, columns]`` (experts first):
+    ``(ids int32 [tokens, top], weights float32 [tokens, top], sigmoid(z[:, shared_at]) or None)``."""
+    lib = library.load()
+    _device_tensor(z, "router logits", torch.float32)
+    _need(z.dim() == 2 and z.shape[1] >= experts and shared_at < z.shape[1], "router logits are [tokens, experts (+ gate)]")
+    n_tokens = z.shape[0]
+    ids = torch.empty((n_tokens, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((n_tokens, top), dtype=torch.float32, device=z.device)
+    shared = torch.empty((n_tokens,), dtype=torch.float32, device=z.device) if shared_at >= 0 else None
+    _check(lib.mll_moe_route(_ptr(z), ctypes.c_int64(z.shape[1]), n_tokens, experts, top, int(softmax_scores), int(renormalize),
+                             int(shared_at), _ptr(ids), _ptr(weights), _ptr(shared), _stream()), lib)
+    return ids, weights, shared
+
+
+MOE_PAIRS_A_LAUNCH = 65535
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
+                weight_on_input: bool, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Every (token, choice) pair through its expert's gated feed-forward: ``gate_up`` ``[experts, 2 * ff, width]``
+    (gate rows first), ``down`` ``[experts, width, ff]``. Returns float32 ``[top, tokens, width]``, a part per choice,
+    for the reader to add in order (``out``: at least that many leading parts of a larger buffer)."""
+    lib = library.load()
+    _device_tensor(x, "expert input")
+    _device_tensor(gate_up, "experts' gate and up weights", x.dtype)
+    _device_tensor(down, "experts' down weights", x.dtype)
+    _device_tensor(ids, "expert ids", torch.int32)
+    _device_tensor(weights, "expert weights", torch.float32)
+    n_tokens, width = x.shape
+    top = ids.shape[1]
+    experts, double, _ = gate_up.shape
+    ff = double // 2
+    _need(gate_up.shape[2] == width and tuple(down.shape) == (experts, width, ff) and tuple(ids.shape) == (n_tokens, top)
+          and tuple(weights.shape) == (n_tokens, top), "the experts' weights, ids and weights do not fit the input")
+    if out is None:
+        out = torch.empty((top, n_tokens, width), dtype=torch.float32, device=x.device)
+    _device_tensor(out, "experts' output", torch.float32)
+    _need(out.dim() == 3 and out.shape[0] >= top and tuple(out.shape[1:]) == (n_tokens, width), "the output is [parts >= top, tokens, width]")
+    act = torch.empty((n_tokens * top, ff), dtype=x.dtype, device=x.device)
+    _need(n_tokens * top <= MOE_PAIRS_A_LAUNCH, "too many (token, expert) pairs for one launch")
+    _check(lib.mll_moe_gate_up(_ptr(x), _ptr(ids), _ptr(weights), top, _ptr(gate_up), _ptr(act), _code(x.dtype), n_tokens, width, ff,
+                               int(weight_on_input), _stream()), lib)
+    _check(lib.mll_moe_down(_ptr(act), _ptr(ids), _ptr(weights), top, _ptr(down), _ptr(out), _code(x.dtype), n_tokens, width, ff,
+                            int(weight_on_input), _stream()), lib)
+    return out
+
+
+def scale_rows(values: torch.Tensor, factor: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[t] = factor[t] * values[t]`` in float32; ``values`` may be parts ``[parts, tokens, width]``, added in order first."""
+    lib = library.load()
+    n_parts, part_stride = _parts_of(values, "values")
+    _device_tensor(factor, "row factors", torch.float32)
+    _device_tensor(out, "scaled rows", torch.float32)
+    n_tokens, width = values.shape[-2], values.shape[-1]
+    _need(tuple(out.shape) == (n_tokens, width) and factor.shape[0] >= n_tokens, "out is [tokens, width], one factor a token")
+    _check(lib.mll_scale_rows(_ptr(values), n_parts, ctypes.c_int64(part_stride), _ptr(factor), _ptr(out), n_tokens, width, _stream()), lib)
+    return out

@@ -1,12 +1,13 @@
-from . import attention, bias_attention, block, feedforward, linear_attention, model, norm, parallel, position, streams  # noqa: F401  (register the built-in kinds)
-from .base import (CacheNeed, CompositeNeed, PagedKeyValueNeed, FeedForward, INT_TABLE, MATRIX, Mixer, Norm, PagedKVNeed, Part, PositionEncoding, Runtime,
+from . import (attention, bias_attention, block, experts, feedforward, latent_attention, linear_attention, model, norm, parallel, position,
+               recurrent, streams)  # noqa: F401  (register the built-in kinds)
+from .base import (CacheNeed, CompositeNeed, PagedKeyValueNeed, PagedLatentNeed, FeedForward, INT_TABLE, MATRIX, Mixer, Norm, PagedKVNeed, Part, PositionEncoding, Runtime,
                    StateNeed, TensorDecl, VECTOR)
 from .block import Block, PreNormBlock, build_block, register_arrangement
 from .model import Model
 from .registry import build_part, register_part, registered_kinds, unregister_part
 from .spec import LayerSpec, ModelSpec, PartSpec, RunEntry, in_order
 
-__all__ = ["CacheNeed", "CompositeNeed", "PagedKeyValueNeed", "FeedForward", "INT_TABLE", "MATRIX", "Mixer", "Norm", "PagedKVNeed", "Part", "PositionEncoding",
+__all__ = ["CacheNeed", "CompositeNeed", "PagedKeyValueNeed", "PagedLatentNeed", "FeedForward", "INT_TABLE", "MATRIX", "Mixer", "Norm", "PagedKVNeed", "Part", "PositionEncoding",
            "Runtime", "StateNeed", "TensorDecl", "VECTOR", "Block", "PreNormBlock", "build_block",
            "register_arrangement", "Model", "build_part", "register_part", "registered_kinds",
            "unregister_part", "LayerSpec", "ModelSpec", "PartSpec", "RunEntry", "in_order"]

@@ -12,7 +12,7 @@ from typing import Dict, Mapping, Optional, Sequence, Tuple, Union
 
 import torch
 
-from ..cache.needs import CacheNeed, CompositeNeed, PagedKVNeed, PagedKeyValueNeed, StateNeed
+from ..cache.needs import CacheNeed, CompositeNeed, PagedKVNeed, PagedKeyValueNeed, PagedLatentNeed, StateNeed
 from .spec import PartSpec
 
 MATRIX = "matrix"   # a float matrix or table: float32 stays float32, bfloat16 stays bfloat16 in a bfloat16 engine

@@ -22,6 +22,9 @@ class RMSNorm(Norm):
         super().__init__(spec, runtime)
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
+        # ``unit_offset``: the file stores the gain's distance from one; the gain ``1 + w`` is formed once, at load,
+        # in float32 (the sum a float32 evaluation of ``x * (1 + w)`` forms for every element).
+        self.unit_offset = bool(spec.params.get("unit_offset", False))
         self.weight: Optional[torch.Tensor] = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
@@ -29,6 +32,8 @@ class RMSNorm(Norm):
 
     def bind(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.name("weight")]
+        if self.unit_offset:
+            self.weight = (self.weight.to(torch.float32) + 1.0).contiguous()
 
     def weight_then_factor(self):
         return (self.weight, self.size, self.eps) if self.weight is not None and self.weight.dtype == torch.float32 else None
