@@ -146,9 +146,16 @@ def gated_ff(h: np.ndarray, t: Dict[str, np.ndarray], prefix: str) -> np.ndarray
     return (silu(h @ t[prefix + "gate"].T) * (h @ t[prefix + "up"].T)) @ t[prefix + "down"].T
 
 
-def routed_ff(h: np.ndarray, t: Dict[str, np.ndarray], prefix: str, mlp: dict) -> np.ndarray:
+def routed_ff(h: np.ndarray, t: Dict[str, np.ndarray], prefix: str, mlp: dict, margins: Optional[List[np.ndarray]] = None) -> np.ndarray:
+    """``margins`` collects, per token, how far the last chosen expert's logit lies above the best one not chosen
+    (infinite where every expert is chosen): a token whose margin is tiny may go to another expert in an engine that
+    rounds, and a test of such an engine leaves it out."""
     experts, top = mlp["router"]["experts"], mlp["router"]["top"]
-    scores = sigmoid(h @ t[prefix + "router"].T)
+    z = h @ t[prefix + "router"].T
+    scores = sigmoid(z)
+    if margins is not None:
+        ordered = -np.sort(-z, axis=1)
+        margins.append(ordered[:, top - 1] - ordered[:, top] if top < experts else np.full(h.shape[0], np.inf))
     out = np.zeros_like(h)
     for row in range(h.shape[0]):
         chosen = sorted(range(experts), key=lambda e: (-scores[row, e], e))[:top]
@@ -161,8 +168,9 @@ def routed_ff(h: np.ndarray, t: Dict[str, np.ndarray], prefix: str, mlp: dict) -
 
 # ---- the model ------------------------------------------------------------------------------------------------
 def forward(config: dict, tensors: Dict[str, np.ndarray], tokens: Sequence[int], layers_out: Optional[List[np.ndarray]] = None,
-            rounded_router_input=None) -> np.ndarray:
-    """Logits ``[n, vocab]`` of one sequence run whole. ``layers_out`` collects the residual stream after every layer."""
+            margins: Optional[List[np.ndarray]] = None) -> np.ndarray:
+    """Logits ``[n, vocab]`` of one sequence run whole. ``layers_out`` collects the residual stream after every layer,
+    ``margins`` the routers' margins (``routed_ff``)."""
     t = {name: np.asarray(value, dtype=np.float64) for name, value in tensors.items()}
     eps = config["norm"]["eps"]
     x = t["embed"][np.asarray(tokens, dtype=np.int64)]
@@ -183,9 +191,49 @@ def forward(config: dict, tensors: Dict[str, np.ndarray], tokens: Sequence[int],
         mlp = layer.get("mlp")
         if mlp is not None:
             h = norm_around_zero(x, t[prefix + "norm2"], eps)
-            if rounded_router_input is not None:
-                h = rounded_router_input(h)
-            x = x + (gated_ff(h, t, prefix + "mlp.") if mlp["kind"] == "dense" else routed_ff(h, t, prefix + "mlp.", mlp))
+            x = x + (gated_ff(h, t, prefix + "mlp.") if mlp["kind"] == "dense" else routed_ff(h, t, prefix + "mlp.", mlp, margins))
         if layers_out is not None:
             layers_out.append(x.copy())
     return norm_around_zero(x, t["final.norm"], eps) @ t["head"].T
+
+
+def folded_attention(q_full: np.ndarray, rows: np.ndarray, kv_rank: int, window: int, scale: float, first: int = 0) -> np.ndarray:
+    """The attention as it runs on cached rows: ``q_full`` [n, heads, row] are queries at positions ``first ..``,
+    ``rows`` [first + n, row] one cached row a position (latent, then the shared turned key part); a query at p sees
+    rows p - window + 1 .. p, and the result is the weighted sum of the rows' first ``kv_rank`` entries."""
+    n, heads, _ = q_full.shape
+    out = np.zeros((n, heads, kv_rank))
+    for i in range(n):
+        p = first + i
+        low = max(0, p - window + 1) if window > 0 else 0
+        for head in range(heads):
+            scores = rows[low:p + 1] @ q_full[i, head] * scale
+            weights = np.exp(scores - scores.max())
+            out[i, head] = (weights / weights.sum()) @ rows[low:p + 1, :kv_rank]
+    return out
+
+
+def choose_experts(z: np.ndarray, top: int, softmax: bool = False, renormalize: bool = False):
+    """Per row of router logits: the ``top`` experts with the largest scores (ties: the lower index) and their weights."""
+    if softmax:
+        e = np.exp(z - z.max(axis=-1, keepdims=True))
+        scores = e / e.sum(axis=-1, keepdims=True)
+    else:
+        scores = sigmoid(z)
+    ids = np.zeros((z.shape[0], top), dtype=np.int64)
+    weights = np.zeros((z.shape[0], top))
+    for row in range(z.shape[0]):
+        order = sorted(range(z.shape[1]), key=lambda e: (-z[row, e], e))[:top]
+        ids[row], weights[row] = order, scores[row, order]
+        if renormalize:
+            weights[row] /= weights[row].sum()
+    return ids, weights
+
+
+def generate_greedy(config: dict, tensors: Dict[str, np.ndarray], prompt: Sequence[int], new_tokens: int) -> List[int]:
+    """The first maximum of the last position's logits, appended ``new_tokens`` times; the whole sequence is run again
+    for every token."""
+    tokens = list(prompt)
+    for _ in range(new_tokens):
+        tokens.append(int(np.argmax(forward(config, tensors, tokens)[-1])))
+    return tokens[len(prompt):]
