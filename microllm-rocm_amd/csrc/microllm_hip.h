@@ -383,4 +383,12 @@ int mll_moe_down(const void* act, const int32_t* ids, const float* weights, int 
 int mll_scale_rows(const float* in, int n_parts, int64_t part_stride, const float* factor, float* out, int n_tokens, int width,
                    hipStream_t stream);
 
+// The same as mll_moe_gate_up and mll_moe_down together for many bfloat16 pairs: the pairs are sorted by expert (counts
+// [experts], offsets [experts + 1], order [n_tokens * top]: int32 scratch), their inputs gathered into `sorted`
+// ([pairs][width]), and every expert multiplies its rows in tiles on the matrix units; `act` is [pairs][ff] scratch.
+// width and ff are multiples of 8.
+int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, const void* down,
+                    int32_t* counts, int32_t* offsets, int32_t* order, void* sorted, void* act, float* out, int n_tokens,
+                    int experts, int width, int ff, int weight_on_input, hipStream_t stream);
+
 }  // extern "C"

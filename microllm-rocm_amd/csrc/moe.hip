@@ -158,6 +158,184 @@ scale_rows_kernel(const float* __restrict__ in, int n_parts, int64_t part_stride
     out[at] = value * factor[token];
 }
 
+// ---- many pairs: rows sorted by expert and tiled MFMA products ---------------------------------------------------
+// With many (token, choice) pairs the pairs are put in the order of their experts (stable: a pair keeps its place
+// among its expert's), their inputs are gathered (and multiplied by their weights) into that order, and every expert
+// multiplies its own stretch of rows: a workgroup takes a tile of up to 128 rows of one expert and 128 of its weight's
+// rows, stages both through LDS in steps of 32 of the reduction and forms the products with
+// v_mfma_f32_16x16x32_bf16 (four waves, 64 x 64 each). Which expert a tile belongs to is read from the device-side
+// offsets; the grid has a tile for every case (pairs / 128 + experts), and tiles beyond the last expert's leave at once.
+// A row's sums do not depend on the other rows of its tile.
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(kWave)
+moe_count_kernel(const int32_t* __restrict__ ids, int n_pairs, int32_t* __restrict__ counts) {
+    const int expert = blockIdx.x, lane = threadIdx.x;
+    int count = 0;
+    for (int p = lane; p < n_pairs; p += kWave) count += ids[p] == expert ? 1 : 0;
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) count += __shfl_xor(count, offset, kWave);
+    if (lane == 0) counts[expert] = count;
+}
+
+// offsets[e] = pairs of the experts before e; order[offsets[e] + n] = the n-th pair (ascending) that chose e.
+__global__ void __launch_bounds__(kWave)
+moe_order_kernel(const int32_t* __restrict__ ids, int n_pairs, int experts, const int32_t* __restrict__ counts,
+                 int32_t* __restrict__ offsets, int32_t* __restrict__ order) {
+    const int expert = blockIdx.x, lane = threadIdx.x;
+    int base = 0;
+    for (int e = 0; e < expert; ++e) base += counts[e];
+    if (lane == 0) {
+        offsets[expert] = base;
+        if (expert == experts - 1) offsets[experts] = base + counts[expert];
+    }
+    int running = 0;
+    for (int first = 0; first < n_pairs; first += kWave) {
+        const int p = first + lane;
+        const bool mine = p < n_pairs && ids[p] == expert;
+        const unsigned long long mask = __ballot(mine);
+        if (mine) order[base + running + __popcll(mask & ((1ull << lane) - 1ull))] = p;
+        running += __popcll(mask);
+    }
+}
+
+// sorted[row] = x[token of order[row]] (* weight of the pair), rounded to bfloat16.
+__global__ void __launch_bounds__(256)
+moe_gather_kernel(const bf16* __restrict__ x, const int32_t* __restrict__ order, const float* __restrict__ weights, int top,
+                  bf16* __restrict__ sorted, int width, int weight_on_input) {
+    const int row = blockIdx.x;
+    const int pair = order[row];
+    const float factor = weight_on_input ? weights[pair] : 1.0f;
+    const bf16* from = x + static_cast<int64_t>(pair / top) * width;
+    bf16* to = sorted + static_cast<int64_t>(row) * width;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) to[c] = from_float<bf16>(to_float(from[c]) * factor);
+}
+
+constexpr int kGroupRows = 128, kGroupCols = 128, kGroupStep = 32, kGroupPad = 40;
+
+// GATED: w is [experts][2 * n_half][k] (gate rows, then up rows); a tile holds 64 gate rows and the 64 up rows that
+// belong to them, and out (bfloat16 [pairs][n_half], sorted order) gets silu(gate) * up. Otherwise w is
+// [experts][n_out][k] and out (float32 [top][n_tokens][n_out]) gets the product at the pair's token and choice,
+// times the pair's weight unless that multiplied the input.
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_grouped_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, const int32_t* __restrict__ offsets,
+                   const int32_t* __restrict__ order, const float* __restrict__ weights, int experts, int n_out, int k,
+                   void* __restrict__ out, int top, int n_tokens, int weight_on_input) {
+    __shared__ __attribute__((aligned(16))) bf16 a_tile[kGroupRows * kGroupPad];
+    __shared__ __attribute__((aligned(16))) bf16 w_tile[kGroupCols * kGroupPad];
+    int expert = 0, first_row = 0, rows = 0, before = 0;
+    for (; expert < experts; ++expert) {
+        const int begin = offsets[expert], end = offsets[expert + 1];
+        const int tiles = (end - begin + kGroupRows - 1) / kGroupRows;
+        if (static_cast<int>(blockIdx.y) < before + tiles) {
+            first_row = begin + (blockIdx.y - before) * kGroupRows;
+            rows = min(kGroupRows, end - first_row);
+            break;
+        }
+        before += tiles;
+    }
+    if (rows == 0) return;      // a tile beyond the last expert's (the same for every thread of the workgroup)
+    const int w_rows = GATED ? 2 * n_out : n_out;
+    const bf16* w_expert = w + static_cast<int64_t>(expert) * w_rows * k;
+    const int col0 = blockIdx.x * (GATED ? 64 : kGroupCols);
+    const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
+    const int wm = wave / 2, wn = wave % 2, r = lane % 16, quad = lane / 16;
+
+    // what this thread brings into LDS each step: two 16-byte pieces of the rows' tile and two of the weight's
+    const bf16* a_from[2];
+    const bf16* w_from[2];
+    int lds_at[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int piece = t + i * 256, row = piece / 4, segment = piece % 4;
+        lds_at[i] = row * kGroupPad + segment * 8;
+        a_from[i] = row < rows ? a + static_cast<int64_t>(first_row + row) * k + segment * 8 : nullptr;
+        int w_row;
+        bool live;
+        if (GATED) {
+            const int column = col0 + row % 64;
+            live = column < n_out;
+            w_row = row < 64 ? column : n_out + column;
+        } else {
+            w_row = col0 + row;
+            live = w_row < n_out;
+        }
+        w_from[i] = live ? w_expert + static_cast<int64_t>(w_row) * k + segment * 8 : nullptr;
+    }
+    floatx4_t acc[4][4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = floatx4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    int w_base[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) w_base[nt] = GATED ? (nt < 2 ? wn * 32 + nt * 16 : 64 + wn * 32 + (nt - 2) * 16) : wn * 64 + nt * 16;
+
+    uint4 a_next[2], w_next[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int segment = (t + i * 256) % 4;
+            const bool in_k = k0 + segment * 8 < k;        // k is a multiple of 8: a piece is whole or absent
+            a_next[i] = (a_from[i] != nullptr && in_k) ? *reinterpret_cast<const uint4*>(a_from[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
+            w_next[i] = (w_from[i] != nullptr && in_k) ? *reinterpret_cast<const uint4*>(w_from[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < k; k0 += kGroupStep) {
+        __syncthreads();        // the step before has read its tiles
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *reinterpret_cast<uint4*>(a_tile + lds_at[i]) = a_next[i];
+            *reinterpret_cast<uint4*>(w_tile + lds_at[i]) = w_next[i];
+        }
+        __syncthreads();
+        if (k0 + kGroupStep < k) fetch(k0 + kGroupStep);      // on its way while this step's products run
+        bf16x8_t a_piece[4], w_piece[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+            a_piece[mt] = *reinterpret_cast<const bf16x8_t*>(a_tile + (wm * 64 + mt * 16 + r) * kGroupPad + quad * 8);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+            w_piece[nt] = *reinterpret_cast<const bf16x8_t*>(w_tile + (w_base[nt] + r) * kGroupPad + quad * 8);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_piece[nt], a_piece[mt], acc[mt][nt], 0, 0, 0);
+    }
+    // acc[mt][nt][i] of lane (r, quad): row wm * 64 + mt * 16 + r of the tile, weight row w_base[nt] + quad * 4 + i
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int row = wm * 64 + mt * 16 + r;
+        if (row >= rows) continue;
+        if (GATED) {
+            bf16* to = static_cast<bf16*>(out) + static_cast<int64_t>(first_row + row) * n_out;
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int column = col0 + wn * 32 + nt * 16 + quad * 4 + i;
+                    const float g = acc[mt][nt][i], u = acc[mt][nt + 2][i];
+                    if (column < n_out) to[column] = from_float<bf16>(g / (1.0f + expf(-g)) * u);
+                }
+        } else {
+            const int pair = order[first_row + row];
+            const float factor = weight_on_input ? 1.0f : weights[pair];
+            float* to = static_cast<float*>(out) + (static_cast<int64_t>(pair % top) * n_tokens + pair / top) * n_out;
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int column = col0 + w_base[nt] + quad * 4 + i;
+                    if (column < n_out) to[column] = acc[mt][nt][i] * factor;
+                }
+        }
+    }
+}
+
 }  // namespace mll
 
 using namespace mll;
@@ -222,6 +400,29 @@ int mll_scale_rows(const float* in, int n_parts, int64_t part_stride, const floa
     if (n_tokens == 0) return 0;
     scale_rows_kernel<<<dim3((width + 255) / 256, n_tokens), 256, 0, stream>>>(in, n_parts, part_stride, factor, out, width);
     return check_launch("scale_rows");
+}
+
+int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int top, const void* gate_up, const void* down,
+                    int32_t* counts, int32_t* offsets, int32_t* order, void* sorted, void* act, float* out, int n_tokens,
+                    int experts, int width, int ff, int weight_on_input, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens > 0 && top > 0 && experts > 0 && width > 0 && ff > 0, "moe_grouped: sizes must be positive");
+    MLL_REQUIRE(width % 8 == 0 && ff % 8 == 0, "moe_grouped: widths must be multiples of 8");
+    const int64_t pairs = static_cast<int64_t>(n_tokens) * top;
+    MLL_REQUIRE(pairs < (1 << 30), "moe_grouped: too many (token, expert) pairs");
+    const int n_pairs = static_cast<int>(pairs);
+    moe_count_kernel<<<experts, kWave, 0, stream>>>(ids, n_pairs, counts);
+    moe_order_kernel<<<experts, kWave, 0, stream>>>(ids, n_pairs, experts, counts, offsets, order);
+    moe_gather_kernel<<<n_pairs, 256, 0, stream>>>(static_cast<const bf16*>(x), order, weights, top, static_cast<bf16*>(sorted), width,
+                                                  weight_on_input);
+    const int tiles = (n_pairs + kGroupRows - 1) / kGroupRows + experts;
+    MLL_REQUIRE(tiles < 65536, "moe_grouped: too many tiles of rows for one launch");
+    moe_grouped_kernel<true><<<dim3((ff + 63) / 64, tiles), 256, 0, stream>>>(
+        static_cast<const bf16*>(sorted), static_cast<const bf16*>(gate_up), offsets, order, weights, experts, ff, width, act, top,
+        n_tokens, weight_on_input);
+    moe_grouped_kernel<false><<<dim3((width + kGroupCols - 1) / kGroupCols, tiles), 256, 0, stream>>>(
+        static_cast<const bf16*>(act), static_cast<const bf16*>(down), offsets, order, weights, experts, width, ff, out, top, n_tokens,
+        weight_on_input);
+    return check_launch("moe_grouped");
 }
 
 }  // extern "C"

@@ -1464,11 +1464,16 @@ def moe_route(z: torch.Tensor, experts: int, top: int, softmax_scores: bool = Fa
 MOE_PAIRS_A_LAUNCH = 65535
 
 
+MOE_GROUPED_PAIRS = 64      # from this many (token, choice) pairs on, bfloat16 experts multiply their rows in tiles
+
+
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
-                weight_on_input: bool, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                weight_on_input: bool, out: Optional[torch.Tensor] = None, grouped: Optional[bool] = None) -> torch.Tensor:
     """Every (token, choice) pair through its expert's gated feed-forward: ``gate_up`` ``[experts, 2 * ff, width]``
     (gate rows first), ``down`` ``[experts, width, ff]``. Returns float32 ``[top, tokens, width]``, a part per choice,
-    for the reader to add in order (``out``: at least that many leading parts of a larger buffer)."""
+    for the reader to add in order (``out``: at least that many leading parts of a larger buffer). ``grouped``: the
+    pairs sorted by expert and multiplied in tiles on the matrix units (bfloat16, widths in steps of 8) instead of
+    one reading of the expert's weights a pair; by default by the number of pairs."""
     lib = library.load()
     _device_tensor(x, "expert input")
     _device_tensor(gate_up, "experts' gate and up weights", x.dtype)
@@ -1486,6 +1491,17 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_
     _device_tensor(out, "experts' output", torch.float32)
     _need(out.dim() == 3 and out.shape[0] >= top and tuple(out.shape[1:]) == (n_tokens, width), "the output is [parts >= top, tokens, width]")
     act = torch.empty((n_tokens * top, ff), dtype=x.dtype, device=x.device)
+    if grouped is None:
+        grouped = x.dtype == torch.bfloat16 and n_tokens * top >= MOE_GROUPED_PAIRS and width % 8 == 0 and ff % 8 == 0
+    if grouped:
+        _need(x.dtype == torch.bfloat16 and width % 8 == 0 and ff % 8 == 0, "the tiled experts take bfloat16 and widths in steps of 8")
+        scratch = torch.empty((2 * experts + 1 + n_tokens * top,), dtype=torch.int32, device=x.device)
+        counts, offsets, order = scratch[:experts], scratch[experts:2 * experts + 1], scratch[2 * experts + 1:]
+        in_order = torch.empty((n_tokens * top, width), dtype=x.dtype, device=x.device)
+        _check(lib.mll_moe_grouped(_ptr(x), _ptr(ids), _ptr(weights), top, _ptr(gate_up), _ptr(down), ctypes.c_void_p(counts.data_ptr()),
+                                   ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()), _ptr(in_order), _ptr(act),
+                                   _ptr(out), n_tokens, experts, width, ff, int(weight_on_input), _stream()), lib)
+        return out
     _need(n_tokens * top <= MOE_PAIRS_A_LAUNCH, "too many (token, expert) pairs for one launch")
     _check(lib.mll_moe_gate_up(_ptr(x), _ptr(ids), _ptr(weights), top, _ptr(gate_up), _ptr(act), _code(x.dtype), n_tokens, width, ff,
                                int(weight_on_input), _stream()), lib)

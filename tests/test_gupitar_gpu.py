@@ -50,7 +50,7 @@ def run_trace(folder, dtype, steps, out_dir, max_tokens, max_requests=4, **optio
 
 
 _plain_logits = {}
-CLOSE_CALL = 0.05       # a router's margin below which a bfloat16 engine may send the token to another expert
+CLOSE_CALL = 0.03       # a router's margin below which a bfloat16 engine may send the token to another expert
 
 
 def plain_logits(config, weights, tokens, with_margins=False):
@@ -67,7 +67,7 @@ def decided(config, weights, tokens, places, dtype):
     if dtype == "float32":
         return np.ones(len(places), dtype=bool)
     margins = plain_logits(config, weights, tokens, with_margins=True)[1][places]
-    assert len(places) < 20 or (margins >= CLOSE_CALL).mean() > 0.7      # the comparison still covers most of the sequence
+    assert len(places) < 40 or (margins >= CLOSE_CALL).mean() > 0.5      # the comparison still covers most of a long sequence
     return margins >= CLOSE_CALL
 
 
@@ -399,6 +399,28 @@ def test_experts_of_every_pair(dtype, on_input):
             want = plain.gated_ff((w * x[token:token + 1]) if on_input else x[token:token + 1], t, "")[0] * (1.0 if on_input else w)
             bound = 1e-5 if dtype == torch.float32 else 0.03
             assert np.abs(parts[choice, token] - want).max() < bound * max(1.0, np.abs(want).max()), (token, choice)
+
+
+@pytest.mark.parametrize("n,width,ff,experts,top", [(300, 64, 40, 6, 2), (70, 200, 136, 3, 3), (513, 96, 264, 16, 1), (5, 48, 8, 4, 2)])
+def test_experts_in_tiles_of_sorted_rows(n, width, ff, experts, top):
+    """The tiled kernels against the kernels that take a pair at a time (which the test above holds against the plain
+    run): experts with no rows, with one, with more than a tile's; widths that do not fill the tiles."""
+    from microllm_rocm_amd.ops import kernels
+    rng = np.random.default_rng(n)
+    x = device(rng.normal(size=(n, width)), torch.bfloat16)
+    gate_up = device(rng.normal(size=(experts, 2 * ff, width)) * 0.2, torch.bfloat16)
+    down = device(rng.normal(size=(experts, width, ff)) * 0.2, torch.bfloat16)
+    busy = rng.permutation(experts)[:max(top, experts - 2)]          # the other experts get no row at all
+    ids = np.stack([rng.permutation(busy)[:top] for _ in range(n)])
+    ids[0, 0] = busy[0]
+    weights = device(rng.uniform(0.2, 1.5, size=(n, top)))
+    for on_input in (True, False):
+        one_by_one = kernels.moe_experts(x, device(ids, torch.int32), weights, gate_up, down, on_input, grouped=False)
+        tiled = kernels.moe_experts(x, device(ids, torch.int32), weights, gate_up, down, on_input, grouped=True)
+        scale = float(one_by_one.abs().max())
+        assert float((tiled - one_by_one).abs().max()) < 0.02 * scale      # the intermediate is rounded to bfloat16 from sums in another order
+        again = kernels.moe_experts(x[:n // 2 + 1], device(ids[:n // 2 + 1], torch.int32), weights[:n // 2 + 1], gate_up, down, on_input, grouped=True)
+        assert torch.equal(again, tiled[:, :n // 2 + 1])      # a row does not depend on the rows beside it
 
 
 # ---- the engine ---------------------------------------------------------------------------------------------------
