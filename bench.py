@@ -69,10 +69,41 @@ DESIGN_SIZES = {
 DESIGN_VOCAB = 32768
 
 
-def design_configs(size: dict):
-    """A Siditar configuration of the given layer sizes and the Qwen2 configuration of equal width, heads, head size,
+def gupitar_config(size: dict):
+    """A Gupitar configuration of the given layer sizes: heads of 96 unrotated and 32 rotated query/key dims and 128
+    value dims, cached rows of 192 + 64 elements (the widest the MFMA attention kernels take), windows of 1024, a
+    recurrence as wide as the model in blocks of 128 with four taps; the first layer's feed-forward dense, the others
+    16 experts of a quarter of the feed-forward width, two a token, and a shared expert of half of it (as many active
+    rows a token as the dense one). Layers in turn: attention, recurrence, attention, attention on the rows of the one before."""
+    from microllm_rocm_amd.config.gupitar import (DenseMlpConfig, GupitarConfig, GupitarLayerConfig, LatentAttentionConfig, MoeMlpConfig,
+                                                  RglruConfig)
+    width, ff = size["width"], size["ff"]
+
+    def attention(kv_from=None):
+        return LatentAttentionConfig(heads=size["heads"], dim=96, rot_dim=64, vdim=size["head_dim"], q_rank=width // 2, kv_rank=192,
+                                     scale=160 ** -0.5, window=1024, rot_base=1e6, rot_dims=64, kv_from=kv_from)
+
+    layers = []
+    for index in range(size["layers"]):
+        kind = ("attention", "recurrence", "attention", "borrow")[index % 4]
+        mlp = DenseMlpConfig(ff) if index == 0 else MoeMlpConfig(experts=16, top=2, expert_ff=ff // 4, shared_ff=ff // 2)
+        if kind == "recurrence":
+            layers.append(GupitarLayerConfig("rglru", RglruConfig(width=width, blocks=width // 128, conv=4), mlp))
+        else:
+            layers.append(GupitarLayerConfig("latent_attention", attention(index - 1 if kind == "borrow" else None), mlp))
+    return GupitarConfig(vocab=DESIGN_VOCAB, width=width, norm_eps=1e-6, layers=tuple(layers))
+
+
+def design_configs(size: dict, design: str = "siditar"):
+    """The design's configuration at the given layer sizes and the Qwen2 configuration of equal width, heads, head size,
     feed-forward width, depth and vocabulary."""
     from microllm_rocm_amd import Qwen2Config
+    qwen2 = Qwen2Config(vocab_size=DESIGN_VOCAB, hidden_size=size["width"], num_hidden_layers=size["layers"],
+                        num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["head_dim"],
+                        intermediate_size=size["ff"], max_position_embeddings=32768, rope_theta=1e6, rms_norm_eps=1e-6,
+                        tie_word_embeddings=False)
+    if design == "gupitar":
+        return {"gupitar": gupitar_config(size), "qwen2": qwen2}
     from microllm_rocm_amd.config.siditar import (BiasAttentionConfig, DenseMlpConfig, LinearAttentionConfig,
                                                   ParallelMixerConfig, SiditarConfig, SiditarLayerConfig)
     left = BiasAttentionConfig(heads=size["heads"], kv_heads=size["kv_heads"], dim=size["head_dim"], vdim=size["head_dim"],
@@ -80,15 +111,11 @@ def design_configs(size: dict):
     right = LinearAttentionConfig(heads=size["heads"] // 2, dim=size["head_dim"] // 2, vdim=size["head_dim"], tau=16.0, decay_rank=16)
     layer = SiditarLayerConfig("parallel", ParallelMixerConfig(left, right, 1.0, 1.0), DenseMlpConfig(size["ff"], 7.0))
     siditar = SiditarConfig(vocab=DESIGN_VOCAB, width=size["width"], norm_eps=1e-6, layers=(layer,) * size["layers"], streams=2)
-    qwen2 = Qwen2Config(vocab_size=DESIGN_VOCAB, hidden_size=size["width"], num_hidden_layers=size["layers"],
-                        num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["head_dim"],
-                        intermediate_size=size["ff"], max_position_embeddings=32768, rope_theta=1e6, rms_norm_eps=1e-6,
-                        tie_word_embeddings=False)
     return {"siditar": siditar, "qwen2": qwen2}
 
 
 def compare_designs(args) -> int:
-    """Prefill and decode throughput of the Siditar design beside Qwen2 at equal layer sizes; prints one JSON line."""
+    """Prefill and decode throughput of the chosen design beside Qwen2 at equal layer sizes; prints one JSON line."""
     import torch
     from microllm_rocm_amd import Engine
     from microllm_rocm_amd.engine.benchmark import decode_throughput, prefill_throughput, step_bytes, step_flops
@@ -96,7 +123,7 @@ def compare_designs(args) -> int:
     peak_flops = BF16_PEAK_FLOPS if args.dtype == "bfloat16" else FP32_PEAK_FLOPS
     for name in [part for part in args.design_sizes.split(",") if part]:
         size = DESIGN_SIZES[name]
-        for design, config in design_configs(size).items():
+        for design, config in design_configs(size, args.design).items():
             if args.design_only and design != args.design_only:
                 continue
             per_request = args.context + args.steps + args.warmup + 2 * page_size
@@ -117,12 +144,12 @@ def compare_designs(args) -> int:
             rows.append(row)
             del engine
             torch.cuda.empty_cache()
-    first = next((row for row in rows if row["design"] == "siditar"), rows[0])
-    line = {"metric": "decode tok/s of the Siditar design beside Qwen2 at equal layer sizes", "value": first["decode"]["tok_per_s"],
+    first = next((row for row in rows if row["design"] == args.design), rows[0])
+    line = {"metric": f"decode tok/s of the {args.design.capitalize()} design beside Qwen2 at equal layer sizes", "value": first["decode"]["tok_per_s"],
             "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["decode"]["ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: random weights, uniform-random token ids, caches filled with random keys and values",
-            "config": {"model": f"Siditar and Qwen2 at sizes {args.design_sizes}", "global_batch": args.batch, "seq_len": args.context,
+            "config": {"model": f"{args.design.capitalize()} and Qwen2 at sizes {args.design_sizes}", "global_batch": args.batch, "seq_len": args.context,
                        "vocab": DESIGN_VOCAB, "kv_block_size": page_size, "parallelism": "single GPU"},
             "compare": rows}
     print(json.dumps(line), flush=True)
@@ -155,11 +182,11 @@ def main() -> int:
     parser.add_argument("--no-extras", action="store_true",
                         help="leave out what the default run adds to its line after the main figures: decoding on the 32-bit path "
                              "at batch 8 and the continuous-batching workload at Qwen2-0.5B sizes")
-    parser.add_argument("--design", default=None, choices=["siditar"],
+    parser.add_argument("--design", default=None, choices=["siditar", "gupitar"],
                         help="instead of the default workload: prefill and decode throughput of this design beside Qwen2 at equal "
                              "layer sizes (--design-sizes), random weights; --batch, --context, --prefill-tokens, --steps apply")
     parser.add_argument("--design-sizes", default="1k,2k,4k", help="of " + ", ".join(sorted(DESIGN_SIZES)))
-    parser.add_argument("--design-only", default=None, choices=["siditar", "qwen2"], help="one of the two designs alone (profiles)")
+    parser.add_argument("--design-only", default=None, choices=["siditar", "gupitar", "qwen2"], help="one of the two designs alone (profiles)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")

@@ -95,42 +95,59 @@ latent_query_kernel(const float* __restrict__ q, int n_tokens, int heads, int di
 }
 
 // ---- a product per head: out[t][h][o] = sum_i x[t][h][i] * w[h][i][o] ----------------------------------------------
-// A workgroup of one wave takes 64 outputs of one head for kHeadProductRows tokens; the tokens' inputs lie in LDS as
-// float32 and every lane walks the inputs in ascending order, so a row's sums do not depend on its neighbours.
-// The weight is stored [head][in][out]: the lanes of a wave read neighbouring outputs. Optionally the result is
-// multiplied by sigmoid(gate[t][h * n_out + o]) (float32 rows, gate_stride apart).
+// A workgroup of four waves takes 64 outputs of one head for kHeadProductRows tokens. The tokens' inputs lie in LDS as
+// float32; wave s walks the s-th quarter of the inputs (the quarters' bounds follow n_in alone) in ascending order and
+// the four partial sums meet in wave order through LDS: a row's sums do not depend on its neighbours. The weight is
+// stored [head][in][out]: the lanes of a wave read neighbouring outputs. Optionally the result is multiplied by
+// sigmoid(gate[t][h * n_out + o]) (float32 rows, gate_stride apart).
 constexpr int kHeadProductRows = 8;
+constexpr int kHeadProductSlices = 4;
 
 template <typename X, typename W, typename O>
-__global__ void __launch_bounds__(kWave)
+__global__ void __launch_bounds__(kHeadProductSlices * kWave)
 head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_head_stride, const W* __restrict__ w,
                     O* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride, const float* __restrict__ gate,
                     int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out) {
-    extern __shared__ float x_rows[];      // [kHeadProductRows][n_in]
+    extern __shared__ float x_rows[];      // [kHeadProductRows][n_in], then [slices - 1][kHeadProductRows][64] partial sums
     const int head = blockIdx.y;
     const int first = blockIdx.z * kHeadProductRows;
     const int rows = min(kHeadProductRows, n_tokens - first);
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
     const int o = blockIdx.x * kWave + lane;
     for (int r = 0; r < rows; ++r) {
         const X* from = x + static_cast<int64_t>(first + r) * x_token_stride + static_cast<int64_t>(head) * x_head_stride;
-        for (int i = lane; i < n_in; i += kWave) x_rows[r * n_in + i] = to_float(from[i]);
+        for (int i = threadIdx.x; i < n_in; i += blockDim.x) x_rows[r * n_in + i] = to_float(from[i]);
     }
+    for (int r = rows; r < kHeadProductRows; ++r)
+        for (int i = threadIdx.x; i < n_in; i += blockDim.x) x_rows[r * n_in + i] = 0.0f;
     __syncthreads();
-    if (o >= n_out) return;
     float acc[kHeadProductRows];
 #pragma unroll
     for (int r = 0; r < kHeadProductRows; ++r) acc[r] = 0.0f;
-    const W* column = w + static_cast<int64_t>(head) * n_in * n_out + o;
-    for (int i = 0; i < n_in; ++i) {
-        const float weight = to_float(column[static_cast<int64_t>(i) * n_out]);
+    const int per_slice = (n_in + kHeadProductSlices - 1) / kHeadProductSlices;
+    const int begin = slice * per_slice, end = min(begin + per_slice, n_in);
+    if (o < n_out) {
+        const W* column = w + static_cast<int64_t>(head) * n_in * n_out + o;
+#pragma unroll 4
+        for (int i = begin; i < end; ++i) {
+            const float weight = to_float(column[static_cast<int64_t>(i) * n_out]);
 #pragma unroll
-        for (int r = 0; r < kHeadProductRows; ++r) acc[r] = fmaf(x_rows[r * n_in + i], weight, acc[r]);
+            for (int r = 0; r < kHeadProductRows; ++r) acc[r] = fmaf(x_rows[r * n_in + i], weight, acc[r]);
+        }
     }
+    float* partial = x_rows + kHeadProductRows * n_in;
+    if (slice > 0) {
+#pragma unroll
+        for (int r = 0; r < kHeadProductRows; ++r) partial[((slice - 1) * kHeadProductRows + r) * kWave + lane] = acc[r];
+    }
+    __syncthreads();
+    if (slice > 0 || o >= n_out) return;
 #pragma unroll
     for (int r = 0; r < kHeadProductRows; ++r) {
         if (r >= rows) break;
         float value = acc[r];
+#pragma unroll
+        for (int other = 1; other < kHeadProductSlices; ++other) value += partial[((other - 1) * kHeadProductRows + r) * kWave + lane];
         if (gate != nullptr) {
             const float g = gate[static_cast<int64_t>(first + r) * gate_stride + static_cast<int64_t>(head) * n_out + o];
             value *= 1.0f / (1.0f + expf(-g));
@@ -248,8 +265,8 @@ int launch_head_product(const void* x, int64_t x_token_stride, int64_t x_head_st
                         int64_t out_token_stride, int64_t out_head_stride, const float* gate, int64_t gate_stride, int n_tokens,
                         int heads, int n_in, int n_out, hipStream_t stream) {
     const dim3 grid((n_out + kWave - 1) / kWave, heads, (n_tokens + kHeadProductRows - 1) / kHeadProductRows);
-    const size_t lds = static_cast<size_t>(kHeadProductRows) * n_in * sizeof(float);
-    head_product_kernel<X, W, O><<<grid, kWave, lds, stream>>>(
+    const size_t lds = (static_cast<size_t>(kHeadProductRows) * n_in + (kHeadProductSlices - 1) * kHeadProductRows * kWave) * sizeof(float);
+    head_product_kernel<X, W, O><<<grid, kHeadProductSlices * kWave, lds, stream>>>(
         static_cast<const X*>(x), x_token_stride, x_head_stride, static_cast<const W*>(w), static_cast<O*>(out),
         out_token_stride, out_head_stride, gate, gate_stride, n_tokens, heads, n_in, n_out);
     return check_launch("head_product");
@@ -315,7 +332,7 @@ int mll_head_product(const void* x, int x_dtype, int64_t x_token_stride, int64_t
                      void* out, int out_dtype, int64_t out_token_stride, int64_t out_head_stride, const float* gate,
                      int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && n_in > 0 && n_out > 0, "head_product: sizes must be positive");
-    MLL_REQUIRE(static_cast<size_t>(kHeadProductRows) * n_in * sizeof(float) <= 64 * 1024, "head_product: inputs wider than 2048 are not supported");
+    MLL_REQUIRE(static_cast<size_t>(kHeadProductRows) * n_in * sizeof(float) <= 56 * 1024, "head_product: inputs wider than 1792 are not supported");
     MLL_REQUIRE(heads < 65536 && (n_tokens + kHeadProductRows - 1) / kHeadProductRows < 65536, "head_product: too many heads or rows for one launch");
     if (n_tokens == 0) return 0;
 #define MLL_HEAD_PRODUCT(X, W, O)                                                                                          \

@@ -391,4 +391,16 @@ int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int
                     int32_t* counts, int32_t* offsets, int32_t* order, void* sorted, void* act, float* out, int n_tokens,
                     int experts, int width, int ff, int weight_on_input, hipStream_t stream);
 
+// mll_rglru_scan for steps with long portions: the recurrence in chunks of 64 tokens (every chunk walked from zero,
+// the state carried from chunk to chunk, every chunk walked again from its start), the same result but for the
+// rounding of the chunks' products. `scratch`: mll_rglru_scan_scratch(n_tokens, n_seqs, width) floats.
+int mll_rglru_scan_chunked(const float* proj, int64_t proj_stride, int x_at, const float* x_bias, int y_at, const float* y_bias,
+                           const float* u, const float* gates, const float* r_bias, const float* i_bias, const float* lam,
+                           float decay_scale, float* state, float* kept, const int32_t* cu_tokens, const int32_t* slots, void* out,
+                           float* scratch, int dtype, int n_tokens, int n_seqs, int width, int blocks, int n_taps, hipStream_t stream);
+int64_t mll_rglru_scan_scratch(int n_tokens, int n_seqs, int width);
+
+// z[t][e] = w[e] . x[t] in float32: x in `dtype`, w float32 [n_out][width] (a router's logits).
+int mll_router_logits(const void* x, int dtype, const float* w, float* z, int n_tokens, int n_out, int width, hipStream_t stream);
+
 }  // extern "C"

@@ -93,6 +93,60 @@ template <> __device__ inline float row_dot<bf16>(const bf16* __restrict__ w, co
     return wave_sum(sum);
 }
 
+// Four rows against the same x at once: four loads on their way a lane instead of one. Each row's sum is formed
+// exactly as row_dot forms it (the same terms in the same order), so a pair's result does not depend on which rows
+// happen to go together.
+template <typename T> __device__ inline void rows_dot4(const T* const (&w)[4], const float* __restrict__ x, int k, int lane, float (&out)[4]);
+
+template <> __device__ inline void rows_dot4<float>(const float* const (&w)[4], const float* __restrict__ x, int k, int lane, float (&out)[4]) {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) out[n] = row_dot<float>(w[n], x, k, lane);
+}
+
+template <> __device__ inline void rows_dot4<bf16>(const bf16* const (&w)[4], const float* __restrict__ x, int k, int lane, float (&out)[4]) {
+    bool fast = (k & 7) == 0;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) fast = fast && (reinterpret_cast<uintptr_t>(w[n]) & 15) == 0;
+    if (!fast) {
+#pragma unroll
+        for (int n = 0; n < 4; ++n) out[n] = row_dot<bf16>(w[n], x, k, lane);
+        return;
+    }
+    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c = lane * 8; c < k; c += kWave * 8) {
+        typedef unsigned int uintx4_t __attribute__((ext_vector_type(4)));
+        uintx4_t raw[4];
+#pragma unroll
+        for (int n = 0; n < 4; ++n) raw[n] = __builtin_nontemporal_load(reinterpret_cast<const uintx4_t*>(w[n] + c));
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            const uint32_t words[4] = {raw[n][0], raw[n][1], raw[n][2], raw[n][3]};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sum[n] = fmaf(__builtin_bit_cast(float, words[i] << 16), x[c + 2 * i], sum[n]);
+                sum[n] = fmaf(__builtin_bit_cast(float, words[i] & 0xffff0000u), x[c + 2 * i + 1], sum[n]);
+            }
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < 4; ++n) out[n] = wave_sum(sum[n]);
+}
+
+// z[t][e] = w[e] . x[t], float32 sums: one workgroup a token, its waves take the rows of w in turn.
+template <typename T>
+__global__ void __launch_bounds__(256)
+router_logits_kernel(const T* __restrict__ x, const float* __restrict__ w, float* __restrict__ z, int n_out, int width) {
+    extern __shared__ float xs[];
+    const int token = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) xs[c] = to_float(x[static_cast<int64_t>(token) * width + c]);
+    __syncthreads();
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    for (int e = wave; e < n_out; e += blockDim.x / kWave) {
+        const float value = row_dot<float>(w + static_cast<int64_t>(e) * width, xs, width, lane);
+        if (lane == 0) z[static_cast<int64_t>(token) * n_out + e] = value;
+    }
+}
+
 constexpr int kExpertWaves = 4;
 constexpr int kExpertRowsAWave = 8;     // outputs a wave forms one after the other
 constexpr int kExpertRowsABlock = kExpertWaves * kExpertRowsAWave;
@@ -113,12 +167,18 @@ moe_gate_up_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids, con
     __syncthreads();
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const T* base = gate_up + static_cast<int64_t>(expert) * 2 * ff * width;
-    for (int n = 0; n < kExpertRowsAWave; ++n) {
+    for (int n = 0; n < kExpertRowsAWave; n += 2) {      // two outputs at a time: their gate and up rows are four rows
         const int f = blockIdx.x * kExpertRowsABlock + wave * kExpertRowsAWave + n;
         if (f >= ff) break;
-        const float g = row_dot<T>(base + static_cast<int64_t>(f) * width, xs, width, lane);
-        const float u = row_dot<T>(base + static_cast<int64_t>(ff + f) * width, xs, width, lane);
-        if (lane == 0) act[static_cast<int64_t>(pair) * ff + f] = from_float<T>(g / (1.0f + expf(-g)) * u);
+        const int second = min(f + 1, ff - 1);
+        const T* const rows[4] = {base + static_cast<int64_t>(f) * width, base + static_cast<int64_t>(ff + f) * width,
+                                  base + static_cast<int64_t>(second) * width, base + static_cast<int64_t>(ff + second) * width};
+        float sums[4];
+        rows_dot4<T>(rows, xs, width, lane, sums);
+        if (lane == 0) {
+            act[static_cast<int64_t>(pair) * ff + f] = from_float<T>(sums[0] / (1.0f + expf(-sums[0])) * sums[1]);
+            if (f + 1 < ff) act[static_cast<int64_t>(pair) * ff + f + 1] = from_float<T>(sums[2] / (1.0f + expf(-sums[2])) * sums[3]);
+        }
     }
 }
 
@@ -137,11 +197,20 @@ moe_down_kernel(const T* __restrict__ act, const int32_t* __restrict__ ids, cons
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const T* base = down + static_cast<int64_t>(expert) * width * ff;
     const float factor = weight_on_input ? 1.0f : weights[pair];
-    for (int n = 0; n < kExpertRowsAWave; ++n) {
+    for (int n = 0; n < kExpertRowsAWave; n += 4) {
         const int c = blockIdx.x * kExpertRowsABlock + wave * kExpertRowsAWave + n;
         if (c >= width) break;
-        const float value = row_dot<T>(base + static_cast<int64_t>(c) * ff, as, ff, lane);
-        if (lane == 0) out[(static_cast<int64_t>(choice) * n_tokens + token) * width + c] = value * factor;
+        const T* rows[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) rows[m] = base + static_cast<int64_t>(min(c + m, width - 1)) * ff;
+        const T* const fixed[4] = {rows[0], rows[1], rows[2], rows[3]};
+        float sums[4];
+        rows_dot4<T>(fixed, as, ff, lane, sums);
+        if (lane == 0) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                if (c + m < width) out[(static_cast<int64_t>(choice) * n_tokens + token) * width + c + m] = sums[m] * factor;
+        }
     }
 }
 
@@ -423,6 +492,21 @@ int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int
         static_cast<const bf16*>(act), static_cast<const bf16*>(down), offsets, order, weights, experts, width, ff, out, top, n_tokens,
         weight_on_input);
     return check_launch("moe_grouped");
+}
+
+int mll_router_logits(const void* x, int dtype, const float* w, float* z, int n_tokens, int n_out, int width, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && n_out > 0 && width > 0, "router_logits: sizes must be positive");
+    MLL_REQUIRE(static_cast<size_t>(width) * sizeof(float) <= 64 * 1024, "router_logits: rows wider than 16384 are not supported");
+    if (n_tokens == 0) return 0;
+    const size_t lds = static_cast<size_t>(width) * sizeof(float);
+    if (dtype == kF32) {
+        router_logits_kernel<float><<<n_tokens, 256, lds, stream>>>(static_cast<const float*>(x), w, z, n_out, width);
+    } else if (dtype == kBF16) {
+        router_logits_kernel<bf16><<<n_tokens, 256, lds, stream>>>(static_cast<const bf16*>(x), w, z, n_out, width);
+    } else {
+        return fail("router_logits: unknown dtype");
+    }
+    return check_launch("router_logits");
 }
 
 }  // extern "C"

@@ -88,6 +88,109 @@ rglru_scan_kernel(const float* __restrict__ proj, int64_t proj_stride, int x_at,
     }
 }
 
+// ---- long portions: the recurrence in chunks ---------------------------------------------------------------------
+// S_t = a_t S_(t-1) + b_t is cut into chunks of kScanChunk tokens of one request. First every chunk is walked from
+// S = 0 (its a and b are formed and kept on the way), which gives its product of decays and what it adds; then one
+// thread a (request, channel) carries the state from chunk to chunk; then every chunk is walked again from the state
+// it starts with. The grid has a chunk for every case (tokens / chunk + requests); which request a chunk belongs to is
+// found from cu_tokens on the device, and chunks beyond the last request's leave at once.
+constexpr int kScanChunk = 64;
+
+__device__ inline bool find_chunk(const int32_t* __restrict__ cu_tokens, int n_seqs, int chunk, int* seq, int* first, int* last) {
+    int before = 0;
+    for (int s = 0; s < n_seqs; ++s) {
+        const int begin = cu_tokens[s], end = cu_tokens[s + 1];
+        const int chunks = (end - begin + kScanChunk - 1) / kScanChunk;
+        if (chunk < before + chunks) {
+            *seq = s;
+            *first = begin + (chunk - before) * kScanChunk;
+            *last = min(*first + kScanChunk, end);
+            return true;
+        }
+        before += chunks;
+    }
+    return false;
+}
+
+__global__ void __launch_bounds__(256)
+rglru_chunk_first_kernel(const float* __restrict__ u, const float* __restrict__ gates, const float* __restrict__ r_bias,
+                         const float* __restrict__ i_bias, const float* __restrict__ lam, float decay_scale,
+                         const int32_t* __restrict__ cu_tokens, int n_seqs, float* __restrict__ decay, float* __restrict__ added,
+                         float* __restrict__ chunk_decay, float* __restrict__ chunk_added, int width, int blocks) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    int seq, first, last;
+    if (c >= width || !find_chunk(cu_tokens, n_seqs, blockIdx.y, &seq, &first, &last)) return;
+    const int size = width / blocks;
+    const int gate_at = (c / size) * 2 * size + c % size;
+    const float rb = r_bias ? r_bias[c] : 0.0f, ib = i_bias ? i_bias[c] : 0.0f;
+    const float rate = -decay_scale * softplus_f(lam[c]);
+    float product = 1.0f, s = 0.0f;
+    for (int token = first; token < last; ++token) {
+        const float* g = gates + static_cast<int64_t>(token) * 2 * width + gate_at;
+        const float r = sigmoid_f(g[0] + rb), i = sigmoid_f(g[size] + ib);
+        const float log_a = rate * r;
+        const float a = expf(log_a);
+        const float b = sqrtf(-expm1f(2.0f * log_a)) * (i * u[static_cast<int64_t>(token) * width + c]);
+        decay[static_cast<int64_t>(token) * width + c] = a;
+        added[static_cast<int64_t>(token) * width + c] = b;
+        product *= a;
+        s = fmaf(a, s, b);
+    }
+    chunk_decay[static_cast<int64_t>(blockIdx.y) * width + c] = product;
+    chunk_added[static_cast<int64_t>(blockIdx.y) * width + c] = s;
+}
+
+// One thread a (request, channel): the state each of the request's chunks starts with (written over chunk_added),
+// the request's state after the step, and the convolution's newest inputs.
+__global__ void __launch_bounds__(256)
+rglru_chunk_carry_kernel(const float* __restrict__ proj, int64_t proj_stride, int x_at, const float* __restrict__ x_bias,
+                         const float* __restrict__ chunk_decay, float* __restrict__ chunk_added, float* __restrict__ state,
+                         float* __restrict__ kept, const int32_t* __restrict__ cu_tokens, const int32_t* __restrict__ slots,
+                         int width, int n_taps) {
+    const int seq = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= width) return;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    if (last <= first) return;
+    int chunk = 0;
+    for (int s = 0; s < seq; ++s) chunk += (cu_tokens[s + 1] - cu_tokens[s] + kScanChunk - 1) / kScanChunk;
+    const int slot = slots[seq];
+    float s = state[static_cast<int64_t>(slot) * width + c];
+    for (int begin = first; begin < last; begin += kScanChunk, ++chunk) {
+        const int64_t at = static_cast<int64_t>(chunk) * width + c;
+        const float starts_with = s;
+        s = fmaf(chunk_decay[at], s, chunk_added[at]);
+        chunk_added[at] = starts_with;
+    }
+    state[static_cast<int64_t>(slot) * width + c] = s;
+    const int before = n_taps - 1, count = last - first;
+    float* tail = kept + static_cast<int64_t>(slot) * before * width;
+    for (int n = 0; n < before; ++n) {
+        const int back = before - n;
+        float value;
+        if (back <= count) value = proj[static_cast<int64_t>(last - back) * proj_stride + x_at + c] + (x_bias ? x_bias[c] : 0.0f);
+        else value = tail[static_cast<int64_t>(before - (back - count)) * width + c];
+        tail[static_cast<int64_t>(n) * width + c] = value;
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+rglru_chunk_second_kernel(const float* __restrict__ proj, int64_t proj_stride, int y_at, const float* __restrict__ y_bias,
+                          const float* __restrict__ decay, const float* __restrict__ added, const float* __restrict__ chunk_start,
+                          const int32_t* __restrict__ cu_tokens, int n_seqs, T* __restrict__ out, int width) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    int seq, first, last;
+    if (c >= width || !find_chunk(cu_tokens, n_seqs, blockIdx.y, &seq, &first, &last)) return;
+    float s = chunk_start[static_cast<int64_t>(blockIdx.y) * width + c];
+    const float yb = y_bias ? y_bias[c] : 0.0f;
+    for (int token = first; token < last; ++token) {
+        const int64_t at = static_cast<int64_t>(token) * width + c;
+        s = fmaf(decay[at], s, added[at]);
+        out[at] = from_float<T>(s * gelu_tanh_f(proj[static_cast<int64_t>(token) * proj_stride + y_at + c] + yb));
+    }
+}
+
 }  // namespace mll
 
 using namespace mll;
@@ -134,6 +237,44 @@ int mll_rglru_scan(const float* proj, int64_t proj_stride, int x_at, const float
         return fail("rglru_scan: unknown dtype");
     }
     return check_launch("rglru_scan");
+}
+
+int mll_rglru_scan_chunked(const float* proj, int64_t proj_stride, int x_at, const float* x_bias, int y_at, const float* y_bias,
+                           const float* u, const float* gates, const float* r_bias, const float* i_bias, const float* lam,
+                           float decay_scale, float* state, float* kept, const int32_t* cu_tokens, const int32_t* slots, void* out,
+                           float* scratch, int dtype, int n_tokens, int n_seqs, int width, int blocks, int n_taps, hipStream_t stream) {
+    MLL_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && width > 0 && blocks > 0 && width % blocks == 0 && n_taps >= 1,
+                "rglru_scan_chunked: the width must divide into blocks");
+    MLL_REQUIRE(n_taps == 1 || kept != nullptr, "rglru_scan_chunked: a convolution of several taps needs the kept inputs");
+    MLL_REQUIRE(scratch != nullptr, "rglru_scan_chunked: scratch of mll_rglru_scan_scratch floats is needed");
+    if (n_seqs == 0 || n_tokens == 0) return 0;
+    const int chunks = (n_tokens + kScanChunk - 1) / kScanChunk + n_seqs;
+    MLL_REQUIRE(n_seqs < 65536 && chunks < 65536, "rglru_scan_chunked: too many requests or chunks for one launch");
+    float* decay = scratch;
+    float* added = decay + static_cast<int64_t>(n_tokens) * width;
+    float* chunk_decay = added + static_cast<int64_t>(n_tokens) * width;
+    float* chunk_added = chunk_decay + static_cast<int64_t>(chunks) * width;
+    const int threads = width >= 256 ? 256 : 64;
+    const dim3 by_chunk((width + threads - 1) / threads, chunks), by_request((width + threads - 1) / threads, n_seqs);
+    rglru_chunk_first_kernel<<<by_chunk, threads, 0, stream>>>(u, gates, r_bias, i_bias, lam, decay_scale, cu_tokens, n_seqs, decay, added,
+                                                              chunk_decay, chunk_added, width, blocks);
+    rglru_chunk_carry_kernel<<<by_request, threads, 0, stream>>>(proj, proj_stride, x_at, x_bias, chunk_decay, chunk_added, state, kept,
+                                                                cu_tokens, slots, width, n_taps);
+    if (dtype == kF32) {
+        rglru_chunk_second_kernel<float><<<by_chunk, threads, 0, stream>>>(proj, proj_stride, y_at, y_bias, decay, added, chunk_added, cu_tokens,
+                                                                          n_seqs, static_cast<float*>(out), width);
+    } else if (dtype == kBF16) {
+        rglru_chunk_second_kernel<bf16><<<by_chunk, threads, 0, stream>>>(proj, proj_stride, y_at, y_bias, decay, added, chunk_added, cu_tokens,
+                                                                         n_seqs, static_cast<bf16*>(out), width);
+    } else {
+        return fail("rglru_scan_chunked: unknown dtype");
+    }
+    return check_launch("rglru_scan_chunked");
+}
+
+int64_t mll_rglru_scan_scratch(int n_tokens, int n_seqs, int width) {
+    const int64_t chunks = (n_tokens + kScanChunk - 1) / kScanChunk + n_seqs;
+    return 2 * (static_cast<int64_t>(n_tokens) + chunks) * width;
 }
 
 }  // extern "C"

@@ -105,7 +105,7 @@ def prefill_throughput(engine: Engine, tokens: int, repeats: int = 3, seed: int 
             "all_ms": [round(elapsed * 1e3, 3) for elapsed in times]}
 
 
-def weight_bytes(engine: Engine) -> int:
+def weight_bytes(engine: Engine, rows: int = 0) -> int:
     """Bytes of every weight a decode step reads once: all layers, the final norm and the head (an embedding
     table that is not the head's is read one row per token, which is counted apart). A matrix counts once,
     at its own size, whichever of its copies (as stored, packed) the step reads."""
@@ -130,6 +130,9 @@ def weight_bytes(engine: Engine) -> int:
     total += count(model.final_norm.weight) + count(model.head.weight)
     for block in model.blocks:
         for part in block.parts():
+            if rows and hasattr(part, "weight_bytes_read"):     # a part that reads only some of its weights in a step of few rows
+                total += part.weight_bytes_read(rows)
+                continue
             for piece in (part, *part.sub_parts()):
                 total += sum(count(value) for value in vars(piece).values())
     return total
@@ -142,7 +145,7 @@ def step_bytes(engine: Engine, batch: int, context: int) -> int:
         visible = context if group.need.window is None else min(context, group.need.window)
         cache += len(group.entries) * visible * group.need.bytes_per_position(engine.dtype)
     cache += engine.cache.state_bytes() // engine.cache.max_requests
-    return weight_bytes(engine) + batch * cache + engine.model.embedding.bytes_read(batch, context)
+    return weight_bytes(engine, rows=batch) + batch * cache + engine.model.embedding.bytes_read(batch, context)
 
 
 def step_flops(engine: Engine, tokens: int) -> float:

@@ -1414,10 +1414,12 @@ def rglru_conv(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], ta
 def rglru_scan(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], y_at: int, y_bias: Optional[torch.Tensor],
                u: torch.Tensor, gates: torch.Tensor, r_bias: Optional[torch.Tensor], i_bias: Optional[torch.Tensor],
                lam: torch.Tensor, decay_scale: float, state: torch.Tensor, kept: torch.Tensor, cu_tokens: torch.Tensor,
-               slots: torch.Tensor, n_seqs: int, blocks: int, n_taps: int, out_dtype: torch.dtype) -> torch.Tensor:
+               slots: torch.Tensor, n_seqs: int, blocks: int, n_taps: int, out_dtype: torch.dtype,
+               chunked: bool = False) -> torch.Tensor:
     """The gated linear recurrence over every request's tokens of the step, times the gated branch; ``state`` float32
     ``[slots, width]`` and ``kept`` ``[slots, taps - 1, width]`` are read and written at ``slots``. Returns
-    ``[tokens, width]`` in ``out_dtype``."""
+    ``[tokens, width]`` in ``out_dtype``. ``chunked``: the recurrence in chunks of tokens that are walked side by
+    side (for steps with long portions; the same result but for the rounding of the chunks' products)."""
     lib = library.load()
     _device_tensor(proj, "projections", torch.float32)
     _device_tensor(u, "convolution output", torch.float32)
@@ -1438,6 +1440,14 @@ def rglru_scan(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], y_
     _device_tensor(slots, "state slots", torch.int32)
     _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
     out = torch.empty((n_tokens, width), dtype=out_dtype, device=u.device)
+    if chunked:
+        lib.mll_rglru_scan_scratch.restype = ctypes.c_int64
+        scratch = torch.empty((int(lib.mll_rglru_scan_scratch(n_tokens, n_seqs, width)),), dtype=torch.float32, device=u.device)
+        _check(lib.mll_rglru_scan_chunked(_ptr(proj), ctypes.c_int64(proj.shape[1]), x_at, _ptr(x_bias), y_at, _ptr(y_bias), _ptr(u),
+                                          _ptr(gates), _ptr(r_bias), _ptr(i_bias), _ptr(lam), ctypes.c_float(decay_scale), _ptr(state),
+                                          _ptr(kept), _ptr(cu_tokens), _ptr(slots), _ptr(out), _ptr(scratch), _code(out_dtype), n_tokens,
+                                          n_seqs, width, blocks, n_taps, _stream()), lib)
+        return out
     _check(lib.mll_rglru_scan(_ptr(proj), ctypes.c_int64(proj.shape[1]), x_at, _ptr(x_bias), y_at, _ptr(y_bias), _ptr(u), _ptr(gates),
                               _ptr(r_bias), _ptr(i_bias), _ptr(lam), ctypes.c_float(decay_scale), _ptr(state), _ptr(kept),
                               _ptr(cu_tokens), _ptr(slots), _ptr(out), _code(out_dtype), n_seqs, width, blocks, n_taps, _stream()), lib)
@@ -1445,6 +1455,18 @@ def rglru_scan(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], y_
 
 
 # ---- a mixture of experts ------------------------------------------------------------------------------------------
+def router_logits(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``x @ weight.T`` with float32 sums: ``x`` in its own dtype, ``weight`` float32 ``[rows, width]`` with few rows
+    (a router's, and what rides with it)."""
+    lib = library.load()
+    _device_tensor(x, "router input")
+    _device_tensor(weight, "router weight", torch.float32)
+    _need(x.dim() == 2 and weight.dim() == 2 and weight.shape[1] == x.shape[1], "router_logits takes [tokens, width] and [rows, width]")
+    z = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
+    _check(lib.mll_router_logits(_ptr(x), _code(x.dtype), _ptr(weight), _ptr(z), x.shape[0], weight.shape[0], x.shape[1], _stream()), lib)
+    return z
+
+
 def moe_route(z: torch.Tensor, experts: int, top: int, softmax_scores: bool = False, renormalize: bool = False,
               shared_at: int = -1):
     """The ``top`` experts of every token from router logits ``z`` float32 ``[tokens, columns]`` (experts first):

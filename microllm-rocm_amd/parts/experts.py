@@ -44,7 +44,7 @@ class RoutedExperts(FeedForward):
             raise ValueError("score is sigmoid or softmax, weight_on input or output, shared_scale sigmoid or None")
         if not 1 <= self.top <= self.experts:
             raise ValueError("between one and all experts a token")
-        self.route_weight: Optional[Weight] = None
+        self.route_weight: Optional[torch.Tensor] = None
         self.gate_up: Optional[torch.Tensor] = None
         self.down: Optional[torch.Tensor] = None
         self.shared_gate_up: Optional[Weight] = None
@@ -68,7 +68,7 @@ class RoutedExperts(FeedForward):
         rows = [tensors[self.name("router")]]
         if self.shared_scale is not None:
             rows.append(tensors[self.name("shared.scale")])
-        self.route_weight = Weight(torch.cat(rows, dim=0).contiguous(), pack=False)
+        self.route_weight = torch.cat(rows, dim=0).contiguous()        # float32 [experts (+ 1), hidden]
         gate_up = down = None
         for expert in range(self.experts):      # every tensor is looked up once: the loader lets go of it then
             gate = tensors[self.name(f"expert{expert}.gate")]
@@ -91,9 +91,17 @@ class RoutedExperts(FeedForward):
         routed = 6.0 * tokens * self.top * self.hidden * self.expert_size
         return super().flops(tokens) + routed + 2.0 * tokens * self.hidden * self.experts
 
+    def weight_bytes_read(self, rows: int) -> int:
+        """Bytes of weights a step of ``rows`` tokens reads at most: the router, the shared expert, and the experts that
+        the rows' choices can reach (each once, where the rows are multiplied in tiles; fewer than a reading a pair)."""
+        element = self.gate_up.element_size()
+        reached = min(self.experts, rows * self.top)
+        total = 4 * self.route_weight.numel() + reached * 3 * self.expert_size * self.hidden * element
+        return total + 3 * self.shared_size * self.hidden * element
+
     def forward(self, x, ctx):
         n_tokens = x.shape[0]
-        z = linear(x, self.route_weight, out_dtype=torch.float32)
+        z = kernels.router_logits(x, self.route_weight)
         ids, weights, shared_factor = kernels.moe_route(z, self.experts, self.top, softmax_scores=self.score == "softmax",
                                                         renormalize=self.renormalize,
                                                         shared_at=self.experts if self.shared_scale is not None else -1)

@@ -28,6 +28,7 @@ class GatedLinearRecurrence(Mixer):
     # A step that is run twice would advance the state twice: the engine, which runs a step once before it captures
     # it, saves the step's state slots before that run and puts them back.
     graph_safe = True
+    LONG_PORTION = 32       # from this many tokens of one request in a step on, the recurrence is walked in chunks side by side
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
         super().__init__(spec, runtime)
@@ -87,7 +88,7 @@ class GatedLinearRecurrence(Mixer):
         kernels.head_product(u.view(n_tokens, self.blocks, self.size), self.gate_weight, gates)
         out = kernels.rglru_scan(proj, self.x_at, self.x_bias, self.y_at, self.y_bias, u, gates.view(n_tokens, 2 * self.width),
                                  self.r_bias, self.i_bias, self.lam, self.decay_scale, state, kept, ctx.cu_tokens, ctx.slots,
-                                 ctx.n_seqs, self.blocks, self.taps, self.runtime.dtype)
+                                 ctx.n_seqs, self.blocks, self.taps, self.runtime.dtype, chunked=ctx.max_count >= self.LONG_PORTION)
         return linear(out, self.o_weight, out_dtype=torch.float32, partials=True)
 
 

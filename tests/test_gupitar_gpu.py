@@ -303,7 +303,7 @@ def test_recurrence_in_steps_with_carried_state():
     for width, blocks, taps in ((96, 3, 4), (70, 5, 2), (64, 1, 1), (130, 2, 3)):
         rng = np.random.default_rng(width)
         size = width // blocks
-        lengths = {"a": 83, "b": 9, "c": 6}
+        lengths = {"a": 213, "b": 9, "c": 6}
         t = {"y.b": rng.normal(size=width), "x.b": rng.normal(size=width), "conv": rng.normal(size=(width, taps)),
              "conv.b": rng.normal(size=width), "ra": rng.normal(size=(blocks, size, size)) * 0.3, "ra.b": rng.normal(size=(blocks, size)),
              "ri": rng.normal(size=(blocks, size, size)) * 0.3, "ri.b": rng.normal(size=(blocks, size)), "lam": rng.normal(size=width)}
@@ -342,16 +342,21 @@ def test_recurrence_in_steps_with_carried_state():
             u = kernels.rglru_conv(proj, width, device(t["x.b"]), device(t["conv"]), device(t["conv.b"]), kept, seq_of_token, cu, slots)
             gates = torch.empty((proj.shape[0], blocks, 2 * size), device="cuda")
             kernels.head_product(u.view(-1, blocks, size), gate_weight, gates)
-            out = kernels.rglru_scan(proj, width, device(t["x.b"]), 0, device(t["y.b"]), u, gates.view(-1, 2 * width), device(t["ra.b"].reshape(-1)),
-                                     device(t["ri.b"].reshape(-1)), device(t["lam"]), 8.0, state, kept, cu, slots, len(names), blocks, taps,
-                                     torch.float32).cpu().numpy()
+            arguments = (proj, width, device(t["x.b"]), 0, device(t["y.b"]), u, gates.view(-1, 2 * width), device(t["ra.b"].reshape(-1)),
+                         device(t["ri.b"].reshape(-1)), device(t["lam"]), 8.0)
+            state_before, kept_before = state.clone(), kept.clone()      # the walk in chunks must leave what the plain walk leaves
+            in_chunks = kernels.rglru_scan(*arguments, state_before, kept_before, cu, slots, len(names), blocks, taps, torch.float32, chunked=True)
+            out = kernels.rglru_scan(*arguments, state, kept, cu, slots, len(names), blocks, taps, torch.float32)
+            assert float((in_chunks - out).abs().max()) < 2e-5 * max(1.0, float(out.abs().max()))
+            assert float((state_before - state).abs().max()) < 2e-5 * max(1.0, float(state.abs().max())) and torch.equal(kept_before, kept)
+            out = out.cpu().numpy()
             first = 0
             for name in names:
                 got[name].append(out[first:first + portions_of[name]])
                 first += portions_of[name]
                 fed[name] += portions_of[name]
 
-        step({"a": 70, "b": 2})
+        step({"a": 200, "b": 2})
         step({"b": 1, "a": 1})
         step({"a": 2, "c": 4, "b": 1})
         for _ in range(5):
