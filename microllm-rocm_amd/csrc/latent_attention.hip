@@ -17,21 +17,24 @@
 namespace mll {
 
 // ---- both latents of a token: norm, rotation, page write ---------------------------------------------------------
-// One wave a (token, which): which 0 is the queries' latent, which 1 the keys' and values'.
+// One workgroup a (token, which): which 0 is the queries' latent, which 1 the keys' and values'.
+constexpr int kPrepareThreads = 256;
+
 template <typename T>
-__global__ void __launch_bounds__(kWave)
+__global__ void __launch_bounds__(kPrepareThreads)
 latent_prepare_kernel(const float* __restrict__ proj, int64_t proj_stride, int q_at, int q_rank, const float* __restrict__ q_weight,
                       int kv_at, int kv_rank, int rot_dim, const float* __restrict__ kv_weight, float eps,
                       const float* __restrict__ cos_sin, const int32_t* __restrict__ slot_mapping, T* __restrict__ q_latent,
                       T* __restrict__ pages, T* __restrict__ k_pages, T* __restrict__ v_pages, int tiled_page_size) {
+    __shared__ float scratch[16];
     const int token = blockIdx.x / 2, which = blockIdx.x % 2;
-    const int lane = threadIdx.x;
+    const int thread = threadIdx.x;
     const float* row = proj + static_cast<int64_t>(token) * proj_stride;
     if (which == 0) {
         float squares = 0.0f;
-        for (int c = lane; c < q_rank; c += kWave) squares = fmaf(row[q_at + c], row[q_at + c], squares);
-        const float factor = 1.0f / sqrtf(wave_sum(squares) / static_cast<float>(q_rank) + eps);
-        for (int c = lane; c < q_rank; c += kWave)
+        for (int c = thread; c < q_rank; c += kPrepareThreads) squares = fmaf(row[q_at + c], row[q_at + c], squares);
+        const float factor = 1.0f / sqrtf(block_sum(squares, scratch) / static_cast<float>(q_rank) + eps);
+        for (int c = thread; c < q_rank; c += kPrepareThreads)
             q_latent[static_cast<int64_t>(token) * q_rank + c] = from_float<T>(row[q_at + c] * factor * q_weight[c]);
         return;
     }
@@ -53,12 +56,12 @@ latent_prepare_kernel(const float* __restrict__ proj, int64_t proj_stride, int q
         }
     };
     float squares = 0.0f;
-    for (int c = lane; c < kv_rank; c += kWave) squares = fmaf(row[kv_at + c], row[kv_at + c], squares);
-    const float factor = 1.0f / sqrtf(wave_sum(squares) / static_cast<float>(kv_rank) + eps);
-    for (int c = lane; c < kv_rank; c += kWave) store(c, row[kv_at + c] * factor * kv_weight[c]);
+    for (int c = thread; c < kv_rank; c += kPrepareThreads) squares = fmaf(row[kv_at + c], row[kv_at + c], squares);
+    const float factor = 1.0f / sqrtf(block_sum(squares, scratch) / static_cast<float>(kv_rank) + eps);
+    for (int c = thread; c < kv_rank; c += kPrepareThreads) store(c, row[kv_at + c] * factor * kv_weight[c]);
     const int half = rot_dim / 2;
     const float* turn = row + kv_at + kv_rank;
-    for (int i = lane; i < half; i += kWave) {
+    for (int i = thread; i < half; i += kPrepareThreads) {
         const float c = cos_sin[(static_cast<int64_t>(token) * half + i) * 2], s = cos_sin[(static_cast<int64_t>(token) * half + i) * 2 + 1];
         store(kv_rank + i, rotate_first(turn[i], turn[i + half], c, s));
         store(kv_rank + i + half, rotate_second(turn[i], turn[i + half], c, s));
@@ -96,63 +99,93 @@ latent_query_kernel(const float* __restrict__ q, int n_tokens, int heads, int di
 
 // ---- a product per head: out[t][h][o] = sum_i x[t][h][i] * w[h][i][o] ----------------------------------------------
 // A workgroup of four waves takes 64 outputs of one head for kHeadProductRows tokens. The tokens' inputs lie in LDS as
-// float32; wave s walks the s-th quarter of the inputs (the quarters' bounds follow n_in alone) in ascending order and
-// the four partial sums meet in wave order through LDS: a row's sums do not depend on its neighbours. The weight is
-// stored [head][in][out]: the lanes of a wave read neighbouring outputs. Optionally the result is multiplied by
-// sigmoid(gate[t][h * n_out + o]) (float32 rows, gate_stride apart).
+// float32, a tile of up to 1024 inputs at a time; wave s walks the s-th quarter of each tile (the bounds follow n_in
+// alone) in ascending order and the four partial sums meet in wave order through LDS: a row's sums do not depend on
+// its neighbours. The weight is stored [head][in][out]: the lanes of a wave read neighbouring outputs. Optionally the
+// result is multiplied by sigmoid(gate[t][h * n_out + o]) (float32 rows, gate_stride apart).
 constexpr int kHeadProductRows = 8;
 constexpr int kHeadProductSlices = 4;
+constexpr int kHeadProductTile = 1024;
 
-template <typename X, typename W, typename O>
-__global__ void __launch_bounds__(kHeadProductSlices * kWave)
+// SLICES 4: four waves, one a quarter (steps of few rows: more loads on their way). SLICES 1: one wave walks the four
+// quarters one after the other into sums of their own (steps of many rows: no exchange, less staging). The same
+// terms are added in the same order either way, so a row's bits do not depend on the step it is in.
+template <typename X, typename W, typename O, int SLICES>
+__global__ void __launch_bounds__(SLICES * kWave)
 head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_head_stride, const W* __restrict__ w,
                     O* __restrict__ out, int64_t out_token_stride, int64_t out_head_stride, const float* __restrict__ gate,
                     int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out) {
-    extern __shared__ float x_rows[];      // [kHeadProductRows][n_in], then [slices - 1][kHeadProductRows][64] partial sums
+    extern __shared__ float x_rows[];      // [kHeadProductRows][tile], then [slices - 1][kHeadProductRows][64] partial sums
+    constexpr int kOwn = kHeadProductSlices / SLICES;       // quarters a thread walks
+    constexpr int kAhead = SLICES == 1 ? 4 : 16;            // weight loads a thread has on their way
     const int head = blockIdx.y;
     const int first = blockIdx.z * kHeadProductRows;
     const int rows = min(kHeadProductRows, n_tokens - first);
     const int lane = threadIdx.x % kWave, slice = threadIdx.x / kWave;
     const int o = blockIdx.x * kWave + lane;
-    for (int r = 0; r < rows; ++r) {
-        const X* from = x + static_cast<int64_t>(first + r) * x_token_stride + static_cast<int64_t>(head) * x_head_stride;
-        for (int i = threadIdx.x; i < n_in; i += blockDim.x) x_rows[r * n_in + i] = to_float(from[i]);
-    }
-    for (int r = rows; r < kHeadProductRows; ++r)
-        for (int i = threadIdx.x; i < n_in; i += blockDim.x) x_rows[r * n_in + i] = 0.0f;
-    __syncthreads();
-    float acc[kHeadProductRows];
+    const int tile = min(n_in, kHeadProductTile);      // the inputs pass through LDS a tile at a time
+    float acc[kOwn][kHeadProductRows];
 #pragma unroll
-    for (int r = 0; r < kHeadProductRows; ++r) acc[r] = 0.0f;
-    const int per_slice = (n_in + kHeadProductSlices - 1) / kHeadProductSlices;
-    const int begin = slice * per_slice, end = min(begin + per_slice, n_in);
-    if (o < n_out) {
-        const W* column = w + static_cast<int64_t>(head) * n_in * n_out + o;
-#pragma unroll 4
-        for (int i = begin; i < end; ++i) {
-            const float weight = to_float(column[static_cast<int64_t>(i) * n_out]);
+    for (int q = 0; q < kOwn; ++q)
 #pragma unroll
-            for (int r = 0; r < kHeadProductRows; ++r) acc[r] = fmaf(x_rows[r * n_in + i], weight, acc[r]);
+        for (int r = 0; r < kHeadProductRows; ++r) acc[q][r] = 0.0f;
+    const W* column = w + static_cast<int64_t>(head) * n_in * n_out + min(o, n_out - 1);
+    for (int i0 = 0; i0 < n_in; i0 += tile) {
+        const int length = min(tile, n_in - i0);
+        __syncthreads();        // the tile before has been read
+        for (int r = 0; r < kHeadProductRows; ++r) {
+            const X* from = x + static_cast<int64_t>(first + min(r, rows - 1)) * x_token_stride + static_cast<int64_t>(head) * x_head_stride + i0;
+            for (int i = threadIdx.x; i < length; i += blockDim.x) x_rows[r * tile + i] = r < rows ? to_float(from[i]) : 0.0f;
+        }
+        __syncthreads();
+        const int per_slice = (length + kHeadProductSlices - 1) / kHeadProductSlices;
+#pragma unroll
+        for (int q = 0; q < kOwn; ++q) {
+            const int quarter = SLICES == 1 ? q : slice;
+            const int begin = quarter * per_slice, end = min(begin + per_slice, length);
+#pragma unroll kAhead
+            for (int i = begin; i < end; ++i) {      // (unrolled so that a thread's loads of the weight are on their way together)
+                const float weight = to_float(column[static_cast<int64_t>(i0 + i) * n_out]);
+#pragma unroll
+                for (int r = 0; r < kHeadProductRows; ++r) acc[q][r] = fmaf(x_rows[r * tile + i], weight, acc[q][r]);
+            }
         }
     }
-    float* partial = x_rows + kHeadProductRows * n_in;
-    if (slice > 0) {
+    float* partial = x_rows + kHeadProductRows * tile;
+    if (SLICES > 1) {
+        if (slice > 0) {
 #pragma unroll
-        for (int r = 0; r < kHeadProductRows; ++r) partial[((slice - 1) * kHeadProductRows + r) * kWave + lane] = acc[r];
+            for (int r = 0; r < kHeadProductRows; ++r) partial[((slice - 1) * kHeadProductRows + r) * kWave + lane] = acc[0][r];
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (slice > 0 || o >= n_out) return;
 #pragma unroll
     for (int r = 0; r < kHeadProductRows; ++r) {
         if (r >= rows) break;
-        float value = acc[r];
+        float value = acc[0][r];
 #pragma unroll
-        for (int other = 1; other < kHeadProductSlices; ++other) value += partial[((other - 1) * kHeadProductRows + r) * kWave + lane];
+        for (int other = 1; other < kHeadProductSlices; ++other)
+            value += SLICES == 1 ? acc[other % kOwn][r] : partial[((other - 1) * kHeadProductRows + r) * kWave + lane];
         if (gate != nullptr) {
             const float g = gate[static_cast<int64_t>(first + r) * gate_stride + static_cast<int64_t>(head) * n_out + o];
             value *= 1.0f / (1.0f + expf(-g));
         }
         out[static_cast<int64_t>(first + r) * out_token_stride + static_cast<int64_t>(head) * out_head_stride + o] = from_float<O>(value);
+    }
+}
+
+// out[t][h * n + c] = in[h][t][c] * sigmoid(gate[t][h * n + c]): the heads of a batched product side by side, gated.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gate_heads_kernel(const T* __restrict__ in, const float* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
+                  int n_tokens, int heads, int n) {
+    const int token = blockIdx.x;
+    for (int column = threadIdx.x; column < heads * n; column += blockDim.x) {
+        const int head = column / n, c = column % n;
+        float value = to_float(in[(static_cast<int64_t>(head) * n_tokens + token) * n + c]);
+        if (gate != nullptr) value *= 1.0f / (1.0f + expf(-gate[static_cast<int64_t>(token) * gate_stride + column]));
+        out[static_cast<int64_t>(token) * heads * n + column] = from_float<T>(value);
     }
 }
 
@@ -260,15 +293,24 @@ latent_attention_kernel(const T* __restrict__ q_full, const T* __restrict__ page
     }
 }
 
+constexpr int kHeadProductFewRows = 64;     // up to this many tokens a step, four waves share a workgroup's reduction
+
 template <typename X, typename W, typename O>
 int launch_head_product(const void* x, int64_t x_token_stride, int64_t x_head_stride, const void* w, void* out,
                         int64_t out_token_stride, int64_t out_head_stride, const float* gate, int64_t gate_stride, int n_tokens,
                         int heads, int n_in, int n_out, hipStream_t stream) {
     const dim3 grid((n_out + kWave - 1) / kWave, heads, (n_tokens + kHeadProductRows - 1) / kHeadProductRows);
-    const size_t lds = (static_cast<size_t>(kHeadProductRows) * n_in + (kHeadProductSlices - 1) * kHeadProductRows * kWave) * sizeof(float);
-    head_product_kernel<X, W, O><<<grid, kHeadProductSlices * kWave, lds, stream>>>(
-        static_cast<const X*>(x), x_token_stride, x_head_stride, static_cast<const W*>(w), static_cast<O*>(out),
-        out_token_stride, out_head_stride, gate, gate_stride, n_tokens, heads, n_in, n_out);
+    const size_t staged = static_cast<size_t>(kHeadProductRows) * (n_in < kHeadProductTile ? n_in : kHeadProductTile);
+    if (n_tokens <= kHeadProductFewRows) {
+        const size_t lds = (staged + (kHeadProductSlices - 1) * kHeadProductRows * kWave) * sizeof(float);
+        head_product_kernel<X, W, O, kHeadProductSlices><<<grid, kHeadProductSlices * kWave, lds, stream>>>(
+            static_cast<const X*>(x), x_token_stride, x_head_stride, static_cast<const W*>(w), static_cast<O*>(out),
+            out_token_stride, out_head_stride, gate, gate_stride, n_tokens, heads, n_in, n_out);
+    } else {
+        head_product_kernel<X, W, O, 1><<<grid, kWave, staged * sizeof(float), stream>>>(
+            static_cast<const X*>(x), x_token_stride, x_head_stride, static_cast<const W*>(w), static_cast<O*>(out),
+            out_token_stride, out_head_stride, gate, gate_stride, n_tokens, heads, n_in, n_out);
+    }
     return check_launch("head_product");
 }
 
@@ -294,11 +336,11 @@ int mll_latent_prepare(const float* proj, int64_t proj_stride, int q_at, int q_r
     MLL_REQUIRE(n_tokens < (1 << 30), "latent_prepare: too many rows for one launch");
     const unsigned blocks = static_cast<unsigned>(n_tokens) * 2;
     if (dtype == kF32) {
-        latent_prepare_kernel<float><<<blocks, kWave, 0, stream>>>(
+        latent_prepare_kernel<float><<<blocks, kPrepareThreads, 0, stream>>>(
             proj, proj_stride, q_at, q_rank, q_weight, kv_at, kv_rank, rot_dim, kv_weight, eps, cos_sin, slot_mapping,
             static_cast<float*>(q_latent), static_cast<float*>(pages), static_cast<float*>(k_pages), static_cast<float*>(v_pages), tiled_page_size);
     } else if (dtype == kBF16) {
-        latent_prepare_kernel<bf16><<<blocks, kWave, 0, stream>>>(
+        latent_prepare_kernel<bf16><<<blocks, kPrepareThreads, 0, stream>>>(
             proj, proj_stride, q_at, q_rank, q_weight, kv_at, kv_rank, rot_dim, kv_weight, eps, cos_sin, slot_mapping,
             static_cast<bf16*>(q_latent), static_cast<bf16*>(pages), static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), tiled_page_size);
     } else {
@@ -332,7 +374,6 @@ int mll_head_product(const void* x, int x_dtype, int64_t x_token_stride, int64_t
                      void* out, int out_dtype, int64_t out_token_stride, int64_t out_head_stride, const float* gate,
                      int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && heads > 0 && n_in > 0 && n_out > 0, "head_product: sizes must be positive");
-    MLL_REQUIRE(static_cast<size_t>(kHeadProductRows) * n_in * sizeof(float) <= 56 * 1024, "head_product: inputs wider than 1792 are not supported");
     MLL_REQUIRE(heads < 65536 && (n_tokens + kHeadProductRows - 1) / kHeadProductRows < 65536, "head_product: too many heads or rows for one launch");
     if (n_tokens == 0) return 0;
 #define MLL_HEAD_PRODUCT(X, W, O)                                                                                          \
@@ -370,6 +411,20 @@ int mll_latent_attention(const void* q_full, const void* pages, const int32_t* b
         return fail("latent_attention: unknown dtype");
     }
     return check_launch("latent_attention");
+}
+
+int mll_gate_heads(const void* in, const float* gate, int64_t gate_stride, void* out, int dtype, int n_tokens, int heads, int n,
+                   hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && heads > 0 && n > 0, "gate_heads: sizes must be positive");
+    if (n_tokens == 0) return 0;
+    if (dtype == kF32) {
+        gate_heads_kernel<float><<<n_tokens, 256, 0, stream>>>(static_cast<const float*>(in), gate, gate_stride, static_cast<float*>(out), n_tokens, heads, n);
+    } else if (dtype == kBF16) {
+        gate_heads_kernel<bf16><<<n_tokens, 256, 0, stream>>>(static_cast<const bf16*>(in), gate, gate_stride, static_cast<bf16*>(out), n_tokens, heads, n);
+    } else {
+        return fail("gate_heads: unknown dtype");
+    }
+    return check_launch("gate_heads");
 }
 
 }  // extern "C"

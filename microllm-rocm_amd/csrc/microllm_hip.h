@@ -336,6 +336,10 @@ int mll_head_product(const void* x, int x_dtype, int64_t x_token_stride, int64_t
                      void* out, int out_dtype, int64_t out_token_stride, int64_t out_head_stride, const float* gate,
                      int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out, hipStream_t stream);
 
+// out[t][h * n + c] = in[h][t][c] (* sigmoid(gate[t][h * n + c]) with gate, float32 rows gate_stride apart); in and out in `dtype`.
+int mll_gate_heads(const void* in, const float* gate, int64_t gate_stride, void* out, int dtype, int n_tokens, int heads, int n,
+                   hipStream_t stream);
+
 // For every token and head: softmax over the keys j in (p - window, p] (window <= 0: all j <= p) of
 // (q_full[t][h] . pages[slot_j]) * scale, out[t][h] = sum_j weight_j pages[slot_j][:kv_rank]. A token whose
 // seq_of_token is negative is skipped. The order of every sum depends on p and the window alone.
@@ -378,6 +382,10 @@ int mll_moe_gate_up(const void* x, const int32_t* ids, const float* weights, int
 // out[n][t] = Wd_e act[t * top + n] (* weights[t][n] unless weight_on_input): float32 [top][n_tokens][width].
 int mll_moe_down(const void* act, const int32_t* ids, const float* weights, int top, const void* down, float* out, int dtype,
                  int n_tokens, int width, int ff, int weight_on_input, hipStream_t stream);
+
+// The same for n_tokens tokens of an output whose parts hold part_tokens rows each (a launch for some of a step's tokens).
+int mll_moe_down_rows(const void* act, const int32_t* ids, const float* weights, int top, const void* down, float* out, int dtype,
+                      int n_tokens, int part_tokens, int width, int ff, int weight_on_input, hipStream_t stream);
 
 // out[t] = factor[t] * (in[0][t] + in[1][t] + ...), float32; parts part_stride elements apart.
 int mll_scale_rows(const float* in, int n_parts, int64_t part_stride, const float* factor, float* out, int n_tokens, int width,

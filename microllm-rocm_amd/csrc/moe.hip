@@ -132,7 +132,7 @@ template <> __device__ inline void rows_dot4<bf16>(const bf16* const (&w)[4], co
     for (int n = 0; n < 4; ++n) out[n] = wave_sum(sum[n]);
 }
 
-// z[t][e] = w[e] . x[t], float32 sums: one workgroup a token, its waves take the rows of w in turn.
+// z[t][e] = w[e] . x[t], float32 sums: a workgroup takes a token and four rows of w, a wave a row.
 template <typename T>
 __global__ void __launch_bounds__(256)
 router_logits_kernel(const T* __restrict__ x, const float* __restrict__ w, float* __restrict__ z, int n_out, int width) {
@@ -141,10 +141,10 @@ router_logits_kernel(const T* __restrict__ x, const float* __restrict__ w, float
     for (int c = threadIdx.x; c < width; c += blockDim.x) xs[c] = to_float(x[static_cast<int64_t>(token) * width + c]);
     __syncthreads();
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    for (int e = wave; e < n_out; e += blockDim.x / kWave) {
-        const float value = row_dot<float>(w + static_cast<int64_t>(e) * width, xs, width, lane);
-        if (lane == 0) z[static_cast<int64_t>(token) * n_out + e] = value;
-    }
+    const int e = blockIdx.y * (blockDim.x / kWave) + wave;     // a wave a row of w
+    if (e >= n_out) return;
+    const float value = row_dot<float>(w + static_cast<int64_t>(e) * width, xs, width, lane);
+    if (lane == 0) z[static_cast<int64_t>(token) * n_out + e] = value;
 }
 
 constexpr int kExpertWaves = 4;
@@ -444,7 +444,12 @@ int mll_moe_gate_up(const void* x, const int32_t* ids, const float* weights, int
 
 int mll_moe_down(const void* act, const int32_t* ids, const float* weights, int top, const void* down, float* out, int dtype,
                  int n_tokens, int width, int ff, int weight_on_input, hipStream_t stream) {
-    MLL_REQUIRE(n_tokens >= 0 && top > 0 && width > 0 && ff > 0, "moe_down: sizes must be positive");
+    return mll_moe_down_rows(act, ids, weights, top, down, out, dtype, n_tokens, n_tokens, width, ff, weight_on_input, stream);
+}
+
+int mll_moe_down_rows(const void* act, const int32_t* ids, const float* weights, int top, const void* down, float* out, int dtype,
+                      int n_tokens, int part_tokens, int width, int ff, int weight_on_input, hipStream_t stream) {
+    MLL_REQUIRE(n_tokens >= 0 && top > 0 && width > 0 && ff > 0 && part_tokens >= n_tokens, "moe_down: sizes must be positive");
     MLL_REQUIRE(static_cast<int64_t>(n_tokens) * top < 65536, "moe_down: too many (token, expert) pairs for one launch");
     MLL_REQUIRE(static_cast<size_t>(ff) * sizeof(float) <= 64 * 1024, "moe_down: experts wider than 16384 are not supported");
     if (n_tokens == 0) return 0;
@@ -452,10 +457,10 @@ int mll_moe_down(const void* act, const int32_t* ids, const float* weights, int 
     const size_t lds = static_cast<size_t>(ff) * sizeof(float);
     if (dtype == kF32) {
         moe_down_kernel<float><<<grid, kExpertWaves * kWave, lds, stream>>>(
-            static_cast<const float*>(act), ids, weights, top, static_cast<const float*>(down), out, n_tokens, width, ff, weight_on_input);
+            static_cast<const float*>(act), ids, weights, top, static_cast<const float*>(down), out, part_tokens, width, ff, weight_on_input);
     } else if (dtype == kBF16) {
         moe_down_kernel<bf16><<<grid, kExpertWaves * kWave, lds, stream>>>(
-            static_cast<const bf16*>(act), ids, weights, top, static_cast<const bf16*>(down), out, n_tokens, width, ff, weight_on_input);
+            static_cast<const bf16*>(act), ids, weights, top, static_cast<const bf16*>(down), out, part_tokens, width, ff, weight_on_input);
     } else {
         return fail("moe_down: unknown dtype");
     }
@@ -497,12 +502,13 @@ int mll_moe_grouped(const void* x, const int32_t* ids, const float* weights, int
 int mll_router_logits(const void* x, int dtype, const float* w, float* z, int n_tokens, int n_out, int width, hipStream_t stream) {
     MLL_REQUIRE(n_tokens >= 0 && n_out > 0 && width > 0, "router_logits: sizes must be positive");
     MLL_REQUIRE(static_cast<size_t>(width) * sizeof(float) <= 64 * 1024, "router_logits: rows wider than 16384 are not supported");
+    MLL_REQUIRE(n_out <= 4 * 65535, "router_logits: too many rows of w for one launch");
     if (n_tokens == 0) return 0;
     const size_t lds = static_cast<size_t>(width) * sizeof(float);
     if (dtype == kF32) {
-        router_logits_kernel<float><<<n_tokens, 256, lds, stream>>>(static_cast<const float*>(x), w, z, n_out, width);
+        router_logits_kernel<float><<<dim3(n_tokens, (n_out + 3) / 4), 256, lds, stream>>>(static_cast<const float*>(x), w, z, n_out, width);
     } else if (dtype == kBF16) {
-        router_logits_kernel<bf16><<<n_tokens, 256, lds, stream>>>(static_cast<const bf16*>(x), w, z, n_out, width);
+        router_logits_kernel<bf16><<<dim3(n_tokens, (n_out + 3) / 4), 256, lds, stream>>>(static_cast<const bf16*>(x), w, z, n_out, width);
     } else {
         return fail("router_logits: unknown dtype");
     }

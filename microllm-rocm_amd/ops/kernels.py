@@ -1359,6 +1359,24 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate:
     return out
 
 
+def gate_heads(values: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """``[heads, tokens, n]`` (a batched product's result) -> ``[tokens, heads * n]``, times ``sigmoid(gate)`` (float32
+    ``[tokens, heads * n]``, unit column stride) if given."""
+    lib = library.load()
+    _device_tensor(values, "values per head")
+    _need(values.dim() == 3, "values are [heads, tokens, n]")
+    heads, n_tokens, n = values.shape
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and tuple(gate.shape) == (n_tokens, heads * n) and gate.stride(1) == 1,
+              "the gate is float32 [tokens, heads * n] with unit column stride")
+        gate_stride = gate.stride(0)
+    out = torch.empty((n_tokens, heads * n), dtype=values.dtype, device=values.device)
+    _check(lib.mll_gate_heads(_ptr(values), ctypes.c_void_p(gate.data_ptr() if gate is not None else 0), ctypes.c_int64(gate_stride),
+                              _ptr(out), _code(values.dtype), n_tokens, heads, n, _stream()), lib)
+    return out
+
+
 def latent_attention(q_full: torch.Tensor, pages: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
                      positions: torch.Tensor, scale: float, window: int, heads: int, kv_rank: int, rot_dim: int) -> torch.Tensor:
     """Attention of folded queries ``[tokens, heads * (kv_rank + rot_dim)]`` over latent pages ``[page, position, kv_rank
@@ -1524,11 +1542,17 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate_
                                    ctypes.c_void_p(offsets.data_ptr()), ctypes.c_void_p(order.data_ptr()), _ptr(in_order), _ptr(act),
                                    _ptr(out), n_tokens, experts, width, ff, int(weight_on_input), _stream()), lib)
         return out
-    _need(n_tokens * top <= MOE_PAIRS_A_LAUNCH, "too many (token, expert) pairs for one launch")
-    _check(lib.mll_moe_gate_up(_ptr(x), _ptr(ids), _ptr(weights), top, _ptr(gate_up), _ptr(act), _code(x.dtype), n_tokens, width, ff,
-                               int(weight_on_input), _stream()), lib)
-    _check(lib.mll_moe_down(_ptr(act), _ptr(ids), _ptr(weights), top, _ptr(down), _ptr(out), _code(x.dtype), n_tokens, width, ff,
-                            int(weight_on_input), _stream()), lib)
+    step = max(1, MOE_PAIRS_A_LAUNCH // top)       # tokens a launch: its grid has a row of workgroups a pair
+    element = x.element_size()
+    for first in range(0, n_tokens, step):
+        count = min(step, n_tokens - first)
+        here = dict(x=ctypes.c_void_p(x.data_ptr() + first * width * element), ids=ctypes.c_void_p(ids.data_ptr() + first * top * 4),
+                    weights=ctypes.c_void_p(weights.data_ptr() + first * top * 4), act=ctypes.c_void_p(act.data_ptr() + first * top * ff * element))
+        _check(lib.mll_moe_gate_up(here["x"], here["ids"], here["weights"], top, _ptr(gate_up), here["act"], _code(x.dtype), count, width, ff,
+                                   int(weight_on_input), _stream()), lib)
+        # the output keeps its rows n_tokens apart in every part: the launch writes its tokens' rows of each
+        _check(lib.mll_moe_down_rows(here["act"], here["ids"], here["weights"], top, _ptr(down), ctypes.c_void_p(out.data_ptr() + first * width * 4),
+                                     _code(x.dtype), count, n_tokens, width, ff, int(weight_on_input), _stream()), lib)
     return out
 
 

@@ -26,13 +26,14 @@ import torch
 from ..ops import kernels
 from .attention import QueryTilePlanner
 from .base import MATRIX, Mixer, PagedKVNeed, PagedLatentNeed, Runtime, TensorDecl, VECTOR
-from .linear import MEDIUM_ROWS, Weight, linear
+from .linear import MEDIUM_ROWS, Weight, linear, linear_into_stream, takes_unscaled
 from .registry import build_part, register_part
 from .spec import PartSpec
 
 
 class LatentAttention(Mixer):
     graph_safe = True
+    fuses_residual = True
     BATCHED_ROWS = MEDIUM_ROWS     # bfloat16 steps of more rows take the library's batched product for the per-head products
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
@@ -121,11 +122,15 @@ class LatentAttention(Mixer):
     def _per_head(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate=None) -> None:
         kernels.head_product(x, weight, out, gate=gate)
 
-    def forward(self, x, ctx, cache):
+    def takes_unscaled(self, rows: int) -> bool:
+        return takes_unscaled(self.in_weight, rows)
+
+    def forward(self, x, ctx, cache, residual=None):
         view = ctx.paged[cache.group]
         dtype = self.runtime.dtype
         n_tokens = x.shape[0]
-        proj = linear(x, self.in_weight, out_dtype=torch.float32)
+        proj = linear(x, self.in_weight, out_dtype=torch.float32)     # applies the rows' factors where x comes without them
+        x = proj        # (only its device is asked for from here on)
         cos_sin = self.position.table(ctx)
         stored = dict(pages=None, k_pages=None, v_pages=None, tiled_page_size=0)
         if self.owns_kv and self.tiled:
@@ -152,9 +157,16 @@ class LatentAttention(Mixer):
         else:
             weighted = kernels.latent_attention(q_full, cache.rows, view.block_table, ctx.seq_of_token, ctx.positions, self.scale,
                                                 self.window, self.heads, self.kv_rank, self.rot_dim)
-        o = torch.empty((n_tokens, self.heads * self.vdim), dtype=dtype, device=x.device)
         gate = proj[:, self.gate_at:self.gate_at + self.heads * self.vdim] if self.output_gate else None
-        self._per_head(weighted, self.unfold_values, o.view(n_tokens, self.heads, self.vdim), gate=gate)
+        if batched:
+            o = kernels.gate_heads(torch.bmm(weighted.transpose(0, 1), self.unfold_values), gate)
+        else:
+            o = torch.empty((n_tokens, self.heads * self.vdim), dtype=dtype, device=x.device)
+            self._per_head(weighted, self.unfold_values, o.view(n_tokens, self.heads, self.vdim), gate=gate)
+        if residual is not None:
+            begun = linear_into_stream(o, self.o_weight, residual)
+            if begun is not None:
+                return begun
         return linear(o, self.o_weight, out_dtype=torch.float32, partials=True)
 
 

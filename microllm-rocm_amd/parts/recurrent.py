@@ -19,7 +19,7 @@ import torch
 
 from ..ops import kernels
 from .base import CompositeNeed, MATRIX, Mixer, Runtime, StateNeed, TensorDecl, VECTOR
-from .linear import Weight, linear
+from .linear import Weight, linear, linear_into_stream, takes_unscaled
 from .registry import register_part
 from .spec import PartSpec
 
@@ -28,6 +28,7 @@ class GatedLinearRecurrence(Mixer):
     # A step that is run twice would advance the state twice: the engine, which runs a step once before it captures
     # it, saves the step's state slots before that run and puts them back.
     graph_safe = True
+    fuses_residual = True
     LONG_PORTION = 32       # from this many tokens of one request in a step on, the recurrence is walked in chunks side by side
 
     def __init__(self, spec: PartSpec, runtime: Runtime):
@@ -79,16 +80,24 @@ class GatedLinearRecurrence(Mixer):
     def flops(self, tokens: int) -> float:
         return super().flops(tokens) + 2.0 * tokens * self.width * (2 * self.size + self.taps + 8)
 
-    def forward(self, x, ctx, cache):
+    def takes_unscaled(self, rows: int) -> bool:
+        return takes_unscaled(self.in_weight, rows)
+
+    def forward(self, x, ctx, cache, residual=None):
         kept, state = cache.parts[0].state, cache.parts[1].state
         n_tokens = x.shape[0]
-        proj = linear(x, self.in_weight, out_dtype=torch.float32)
+        proj = linear(x, self.in_weight, out_dtype=torch.float32)     # applies the rows' factors where x comes without them
+        x = proj
         u = kernels.rglru_conv(proj, self.x_at, self.x_bias, self.conv, self.conv_bias, kept, ctx.seq_of_token, ctx.cu_tokens, ctx.slots)
         gates = torch.empty((n_tokens, self.blocks, 2 * self.size), dtype=torch.float32, device=x.device)
         kernels.head_product(u.view(n_tokens, self.blocks, self.size), self.gate_weight, gates)
         out = kernels.rglru_scan(proj, self.x_at, self.x_bias, self.y_at, self.y_bias, u, gates.view(n_tokens, 2 * self.width),
                                  self.r_bias, self.i_bias, self.lam, self.decay_scale, state, kept, ctx.cu_tokens, ctx.slots,
                                  ctx.n_seqs, self.blocks, self.taps, self.runtime.dtype, chunked=ctx.max_count >= self.LONG_PORTION)
+        if residual is not None:
+            begun = linear_into_stream(out, self.o_weight, residual)
+            if begun is not None:
+                return begun
         return linear(out, self.o_weight, out_dtype=torch.float32, partials=True)
 
 

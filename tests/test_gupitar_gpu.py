@@ -164,7 +164,7 @@ def test_latents_norm_rotation_and_page_write(q_rank, kv_rank, rot, tiled, dtype
 
 @pytest.mark.parametrize("types", [(torch.float32, torch.float32, torch.float32), (torch.float32, torch.bfloat16, torch.bfloat16),
                                    (torch.bfloat16, torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16, torch.float32)])
-@pytest.mark.parametrize("n,heads,n_in,n_out", [(1, 1, 5, 3), (9, 3, 16, 40), (20, 2, 70, 130)])
+@pytest.mark.parametrize("n,heads,n_in,n_out", [(1, 1, 5, 3), (9, 3, 16, 40), (20, 2, 70, 130), (3, 2, 1500, 70)])
 def test_product_per_head(types, n, heads, n_in, n_out):
     """Views with strides of their own on both sides, a gate, rows that do not fill a workgroup's tile."""
     from microllm_rocm_amd.ops import kernels
@@ -184,10 +184,14 @@ def test_product_per_head(types, n, heads, n_in, n_out):
     kernels.head_product(x_device[:, :, :n_in], device(w, w_type), out[:, :, 2:2 + n_out], gate=gate_device[:, :heads * n_out])
     gated = want * plain.sigmoid(gate[:, :heads * n_out]).reshape(n, heads, n_out)
     assert np.abs(out[:, :, 2:2 + n_out].float().cpu().numpy() - gated).max() < bound * max(1.0, np.abs(want).max())
-    if x_type == torch.float32:       # a row's sums do not depend on the rows beside it
+    if x_type == torch.float32:       # a row's sums do not depend on the rows beside it, nor on which of the two kernels a step's size takes
         alone = torch.zeros((1, heads, n_out), dtype=out_type, device="cuda")
         kernels.head_product(x_device[n - 1:, :, :n_in], device(w, w_type), alone, gate=gate_device[n - 1:, :heads * n_out])
         assert torch.equal(alone[0], out[n - 1, :, 2:2 + n_out])
+        many = torch.zeros((70, heads, n_out), dtype=out_type, device="cuda")
+        kernels.head_product(x_device[n - 1:, :, :n_in].expand(70, heads, n_in), device(w, w_type), many)
+        kernels.head_product(x_device[n - 1:, :, :n_in], device(w, w_type), alone)
+        assert torch.equal(many[69], alone[0]) and torch.equal(many[0], alone[0])
 
 
 def test_queries_are_folded_and_turned():
@@ -210,6 +214,17 @@ def test_queries_are_folded_and_turned():
     assert np.abs(flat.cpu().numpy() - q[:, :, :dim].transpose(1, 0, 2)).max() < 1e-6
     kernels.latent_query(q_device, heads, dim, rot, rank, cos_sin, joined, folded=torch.bmm(flat, device(fold)))
     assert np.abs(joined.cpu().numpy().reshape(n, heads, -1) - want).max() < 2e-5
+
+
+def test_heads_side_by_side_and_gated():
+    from microllm_rocm_amd.ops import kernels
+    rng = np.random.default_rng(8)
+    values, gate = as_bf16(rng.normal(size=(3, 11, 20))), rng.normal(size=(11, 70))
+    want = values.transpose(1, 0, 2).reshape(11, 60)
+    for dtype, bound in ((torch.float32, 1e-6), (torch.bfloat16, 0.02)):
+        assert np.abs(kernels.gate_heads(device(values, dtype), None).float().cpu().numpy() - want).max() == 0.0
+        got = kernels.gate_heads(device(values, dtype), device(gate)[:, 5:65]).float().cpu().numpy()
+        assert np.abs(got - want * plain.sigmoid(gate[:, 5:65])).max() < bound
 
 
 def attention_over_rows(q_full, rows, rank, window, scale, portions_of, mfma, page_size=16):
@@ -404,6 +419,12 @@ def test_experts_of_every_pair(dtype, on_input):
             want = plain.gated_ff((w * x[token:token + 1]) if on_input else x[token:token + 1], t, "")[0] * (1.0 if on_input else w)
             bound = 1e-5 if dtype == torch.float32 else 0.03
             assert np.abs(parts[choice, token] - want).max() < bound * max(1.0, np.abs(want).max()), (token, choice)
+    limit, kernels.MOE_PAIRS_A_LAUNCH = kernels.MOE_PAIRS_A_LAUNCH, 7        # a step of more pairs than a launch takes goes in several
+    try:
+        in_pieces = kernels.moe_experts(device(x, dtype), device(ids, torch.int32), device(weights), device(gate_up, dtype), device(down, dtype), on_input)
+    finally:
+        kernels.MOE_PAIRS_A_LAUNCH = limit
+    assert np.array_equal(in_pieces.cpu().numpy(), parts)
 
 
 @pytest.mark.parametrize("n,width,ff,experts,top", [(300, 64, 40, 6, 2), (70, 200, 136, 3, 3), (513, 96, 264, 16, 1), (5, 48, 8, 4, 2)])
