@@ -119,9 +119,6 @@ class LatentAttention(Mixer):
         per_head = 2.0 * tokens * self.heads * self.kv_rank * (self.dim + self.vdim)
         return super().flops(tokens) + per_head + 2.0 * self.heads * (self.row + self.kv_rank) * pairs
 
-    def _per_head(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, gate=None) -> None:
-        kernels.head_product(x, weight, out, gate=gate)
-
     def takes_unscaled(self, rows: int) -> bool:
         return takes_unscaled(self.in_weight, rows)
 
@@ -130,7 +127,7 @@ class LatentAttention(Mixer):
         dtype = self.runtime.dtype
         n_tokens = x.shape[0]
         proj = linear(x, self.in_weight, out_dtype=torch.float32)     # applies the rows' factors where x comes without them
-        x = proj        # (only its device is asked for from here on)
+        device = proj.device
         cos_sin = self.position.table(ctx)
         stored = dict(pages=None, k_pages=None, v_pages=None, tiled_page_size=0)
         if self.owns_kv and self.tiled:
@@ -140,14 +137,14 @@ class LatentAttention(Mixer):
         cq = kernels.latent_prepare(proj, self.q_at, self.q_rank, self.q_norm, self.kv_at, self.kv_rank, self.rot_dim, self.kv_norm,
                                     self.eps, cos_sin, view.slot_mapping if self.owns_kv else None, dtype, **stored)
         q = linear(cq, self.uq_weight, out_dtype=torch.float32)         # rounded once, after folding and rotation
-        q_full = torch.empty((n_tokens, self.heads * self.row), dtype=dtype, device=x.device)
+        q_full = torch.empty((n_tokens, self.heads * self.row), dtype=dtype, device=device)
         batched = dtype == torch.bfloat16 and n_tokens > self.BATCHED_ROWS
         if batched:
             flat = kernels.latent_query(q, self.heads, self.dim, self.rot_dim, self.kv_rank, cos_sin, q_full, want_flat=True)
             folded = torch.bmm(flat, self.fold_keys)
             kernels.latent_query(q, self.heads, self.dim, self.rot_dim, self.kv_rank, cos_sin, q_full, folded=folded)
         else:
-            self._per_head(q.view(n_tokens, self.heads, self.dim + self.rot_dim)[:, :, :self.dim], self.fold_keys,
+            kernels.head_product(q.view(n_tokens, self.heads, self.dim + self.rot_dim)[:, :, :self.dim], self.fold_keys,
                            q_full.view(n_tokens, self.heads, self.row)[:, :, :self.kv_rank])
             kernels.latent_query(q, self.heads, self.dim, self.rot_dim, self.kv_rank, cos_sin, q_full)
         if self.tiled:
@@ -161,8 +158,8 @@ class LatentAttention(Mixer):
         if batched:
             o = kernels.gate_heads(torch.bmm(weighted.transpose(0, 1), self.unfold_values), gate)
         else:
-            o = torch.empty((n_tokens, self.heads * self.vdim), dtype=dtype, device=x.device)
-            self._per_head(weighted, self.unfold_values, o.view(n_tokens, self.heads, self.vdim), gate=gate)
+            o = torch.empty((n_tokens, self.heads * self.vdim), dtype=dtype, device=device)
+            kernels.head_product(weighted, self.unfold_values, o.view(n_tokens, self.heads, self.vdim), gate=gate)
         if residual is not None:
             begun = linear_into_stream(o, self.o_weight, residual)
             if begun is not None:

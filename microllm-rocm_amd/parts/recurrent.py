@@ -87,9 +87,8 @@ class GatedLinearRecurrence(Mixer):
         kept, state = cache.parts[0].state, cache.parts[1].state
         n_tokens = x.shape[0]
         proj = linear(x, self.in_weight, out_dtype=torch.float32)     # applies the rows' factors where x comes without them
-        x = proj
         u = kernels.rglru_conv(proj, self.x_at, self.x_bias, self.conv, self.conv_bias, kept, ctx.seq_of_token, ctx.cu_tokens, ctx.slots)
-        gates = torch.empty((n_tokens, self.blocks, 2 * self.size), dtype=torch.float32, device=x.device)
+        gates = torch.empty((n_tokens, self.blocks, 2 * self.size), dtype=torch.float32, device=proj.device)
         kernels.head_product(u.view(n_tokens, self.blocks, self.size), self.gate_weight, gates)
         out = kernels.rglru_scan(proj, self.x_at, self.x_bias, self.y_at, self.y_bias, u, gates.view(n_tokens, 2 * self.width),
                                  self.r_bias, self.i_bias, self.lam, self.decay_scale, state, kept, ctx.cu_tokens, ctx.slots,
