@@ -117,7 +117,7 @@ head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_h
                     int64_t gate_stride, int n_tokens, int heads, int n_in, int n_out) {
     extern __shared__ float x_rows[];      // [kHeadProductRows][tile], then [slices - 1][kHeadProductRows][64] partial sums
     constexpr int kOwn = kHeadProductSlices / SLICES;       // quarters a thread walks
-    constexpr int kAhead = SLICES == 1 ? 4 : 16;            // weight loads a thread has on their way
+    constexpr int kAhead = 16;                              // weight loads a thread of the four-wave kernel has on their way
     const int head = blockIdx.y;
     const int first = blockIdx.z * kHeadProductRows;
     const int rows = min(kHeadProductRows, n_tokens - first);
@@ -143,11 +143,26 @@ head_product_kernel(const X* __restrict__ x, int64_t x_token_stride, int64_t x_h
         for (int q = 0; q < kOwn; ++q) {
             const int quarter = SLICES == 1 ? q : slice;
             const int begin = quarter * per_slice, end = min(begin + per_slice, length);
-#pragma unroll kAhead
-            for (int i = begin; i < end; ++i) {      // (unrolled so that a thread's loads of the weight are on their way together)
-                const float weight = to_float(column[static_cast<int64_t>(i0 + i) * n_out]);
+            if constexpr (SLICES == 1) {
+#pragma unroll 4
+                for (int i = begin; i < end; ++i) {
+                    const float weight = to_float(column[static_cast<int64_t>(i0 + i) * n_out]);
 #pragma unroll
-                for (int r = 0; r < kHeadProductRows; ++r) acc[q][r] = fmaf(x_rows[r * tile + i], weight, acc[q][r]);
+                    for (int r = 0; r < kHeadProductRows; ++r) acc[q][r] = fmaf(x_rows[r * tile + i], weight, acc[q][r]);
+                }
+                continue;
+            }
+            for (int i = begin; i < end; i += kAhead) {      // few rows: kAhead loads of the weight are asked for before the first is used
+                W ahead[kAhead];
+#pragma unroll
+                for (int n = 0; n < kAhead; ++n) ahead[n] = column[static_cast<int64_t>(i0 + min(i + n, end - 1)) * n_out];
+#pragma unroll
+                for (int n = 0; n < kAhead; ++n) {
+                    const float weight = i + n < end ? to_float(ahead[n]) : 0.0f;      // past the end: a term of exactly zero
+                    const int at = min(i + n, end - 1);
+#pragma unroll
+                    for (int r = 0; r < kHeadProductRows; ++r) acc[q][r] = fmaf(x_rows[r * tile + at], weight, acc[q][r]);
+                }
             }
         }
     }

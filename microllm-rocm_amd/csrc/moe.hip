@@ -231,7 +231,7 @@ scale_rows_kernel(const float* __restrict__ in, int n_parts, int64_t part_stride
 // With many (token, choice) pairs the pairs are put in the order of their experts (stable: a pair keeps its place
 // among its expert's), their inputs are gathered (and multiplied by their weights) into that order, and every expert
 // multiplies its own stretch of rows: a workgroup takes a tile of up to 128 rows of one expert and 128 of its weight's
-// rows, stages both through LDS in steps of 32 of the reduction and forms the products with
+// rows, stages both through LDS in steps of 64 of the reduction and forms the products with
 // v_mfma_f32_16x16x32_bf16 (four waves, 64 x 64 each). Which expert a tile belongs to is read from the device-side
 // offsets; the grid has a tile for every case (pairs / 128 + experts), and tiles beyond the last expert's leave at once.
 // A row's sums do not depend on the other rows of its tile.
@@ -281,7 +281,7 @@ moe_gather_kernel(const bf16* __restrict__ x, const int32_t* __restrict__ order,
     for (int c = threadIdx.x; c < width; c += blockDim.x) to[c] = from_float<bf16>(to_float(from[c]) * factor);
 }
 
-constexpr int kGroupRows = 128, kGroupCols = 128, kGroupStep = 32, kGroupPad = 40;
+constexpr int kGroupRows = 128, kGroupCols = 128, kGroupStep = 64, kGroupPad = 72;     // rows of a tile lie 144 bytes apart in LDS: 16-byte reads of 16 rows meet no bank twice
 
 // GATED: w is [experts][2 * n_half][k] (gate rows, then up rows); a tile holds 64 gate rows and the 64 up rows that
 // belong to them, and out (bfloat16 [pairs][n_half], sorted order) gets silu(gate) * up. Otherwise w is
@@ -312,13 +312,14 @@ moe_grouped_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, const
     const int t = threadIdx.x, lane = t % kWave, wave = t / kWave;
     const int wm = wave / 2, wn = wave % 2, r = lane % 16, quad = lane / 16;
 
-    // what this thread brings into LDS each step: two 16-byte pieces of the rows' tile and two of the weight's
-    const bf16* a_from[2];
-    const bf16* w_from[2];
-    int lds_at[2];
+    // what this thread brings into LDS each step: four 16-byte pieces of the rows' tile and four of the weight's
+    constexpr int kPieces = kGroupRows * (kGroupStep / 8) / 256;
+    const bf16* a_from[kPieces];
+    const bf16* w_from[kPieces];
+    int lds_at[kPieces];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int piece = t + i * 256, row = piece / 4, segment = piece % 4;
+    for (int i = 0; i < kPieces; ++i) {
+        const int piece = t + i * 256, row = piece / (kGroupStep / 8), segment = piece % (kGroupStep / 8);
         lds_at[i] = row * kGroupPad + segment * 8;
         a_from[i] = row < rows ? a + static_cast<int64_t>(first_row + row) * k + segment * 8 : nullptr;
         int w_row;
@@ -342,11 +343,11 @@ moe_grouped_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, const
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) w_base[nt] = GATED ? (nt < 2 ? wn * 32 + nt * 16 : 64 + wn * 32 + (nt - 2) * 16) : wn * 64 + nt * 16;
 
-    uint4 a_next[2], w_next[2];
+    uint4 a_next[kPieces], w_next[kPieces];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int segment = (t + i * 256) % 4;
+        for (int i = 0; i < kPieces; ++i) {
+            const int segment = (t + i * 256) % (kGroupStep / 8);
             const bool in_k = k0 + segment * 8 < k;        // k is a multiple of 8: a piece is whole or absent
             a_next[i] = (a_from[i] != nullptr && in_k) ? *reinterpret_cast<const uint4*>(a_from[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
             w_next[i] = (w_from[i] != nullptr && in_k) ? *reinterpret_cast<const uint4*>(w_from[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
@@ -356,24 +357,27 @@ moe_grouped_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, const
     for (int k0 = 0; k0 < k; k0 += kGroupStep) {
         __syncthreads();        // the step before has read its tiles
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < kPieces; ++i) {
             *reinterpret_cast<uint4*>(a_tile + lds_at[i]) = a_next[i];
             *reinterpret_cast<uint4*>(w_tile + lds_at[i]) = w_next[i];
         }
         __syncthreads();
         if (k0 + kGroupStep < k) fetch(k0 + kGroupStep);      // on its way while this step's products run
-        bf16x8_t a_piece[4], w_piece[4];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-            a_piece[mt] = *reinterpret_cast<const bf16x8_t*>(a_tile + (wm * 64 + mt * 16 + r) * kGroupPad + quad * 8);
+        for (int half = 0; half < kGroupStep / 32; ++half) {
+            bf16x8_t a_piece[4], w_piece[4];
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-            w_piece[nt] = *reinterpret_cast<const bf16x8_t*>(w_tile + (w_base[nt] + r) * kGroupPad + quad * 8);
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+            for (int mt = 0; mt < 4; ++mt)
+                a_piece[mt] = *reinterpret_cast<const bf16x8_t*>(a_tile + (wm * 64 + mt * 16 + r) * kGroupPad + half * 32 + quad * 8);
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt)
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_piece[nt], a_piece[mt], acc[mt][nt], 0, 0, 0);
+                w_piece[nt] = *reinterpret_cast<const bf16x8_t*>(w_tile + (w_base[nt] + r) * kGroupPad + half * 32 + quad * 8);
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_piece[nt], a_piece[mt], acc[mt][nt], 0, 0, 0);
+        }
     }
     // acc[mt][nt][i] of lane (r, quad): row wm * 64 + mt * 16 + r of the tile, weight row w_base[nt] + quad * 4 + i
 #pragma unroll
