@@ -1459,7 +1459,6 @@ def rglru_scan(proj: torch.Tensor, x_at: int, x_bias: Optional[torch.Tensor], y_
     _need(cu_tokens.shape[0] >= n_seqs + 1 and slots.shape[0] >= n_seqs, "offsets and slots for every request")
     out = torch.empty((n_tokens, width), dtype=out_dtype, device=u.device)
     if chunked:
-        lib.mll_rglru_scan_scratch.restype = ctypes.c_int64
         scratch = torch.empty((int(lib.mll_rglru_scan_scratch(n_tokens, n_seqs, width)),), dtype=torch.float32, device=u.device)
         _check(lib.mll_rglru_scan_chunked(_ptr(proj), ctypes.c_int64(proj.shape[1]), x_at, _ptr(x_bias), y_at, _ptr(y_bias), _ptr(u),
                                           _ptr(gates), _ptr(r_bias), _ptr(i_bias), _ptr(lam), ctypes.c_float(decay_scale), _ptr(state),

@@ -179,6 +179,7 @@ def load() -> ctypes.CDLL:
         raise KernelLibraryError(f"cannot load {path}: {error}") from error
     _library.mll_last_error.restype = ctypes.c_char_p
     _library.mll_sample_workspace.restype = ctypes.c_int64
+    _library.mll_rglru_scan_scratch.restype = ctypes.c_int64
     return _library
 
 

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import plain_gupitar as plain
-from gupitar_tiny import CONFIGS, make_gupitar_folder
+from gupitar_tiny import make_gupitar_folder
 from replay_tools import collect, mixed, portions, prefill_then_decode, round_up, to_lines, whole
 
 pytestmark = pytest.mark.gpu
