@@ -465,6 +465,9 @@ def test_whole_decode_and_portions(tmp_path_factory, tmp_path, which, dtype):
         steps = portions("long", requests["long"], sizes)
         run_trace(folder, dtype, steps, tmp_path / f"portions_{sizes[0]}", max_tokens=192)
         check_against_plain(steps, tmp_path / f"portions_{sizes[0]}", {"long": requests["long"]}, config, weights, dtype)
+    steps = portions("short", requests["short"], [1])       # from its first token on, one token a step
+    run_trace(folder, dtype, steps, tmp_path / "one_by_one", max_tokens=64)
+    check_against_plain(steps, tmp_path / "one_by_one", {"short": requests["short"]}, config, weights, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
